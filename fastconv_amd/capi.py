@@ -1,0 +1,295 @@
+"""ctypes binding of include/fastconv_hip.h (no torch, no numpy compute)."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libfastconv_hip.so")
+
+STAGE_NAMES = ["KernelTran", "InputTran", "TensorGEMM", "OutputTran", "ImplicitGemm", "FilterPack",
+               "FusedGemmOut"]
+
+
+class FastConvError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__("fastconv status %d: %s" % (status, message))
+        self.status = status
+
+
+class ConvShape(C.Structure):
+    _fields_ = [(n, C.c_int) for n in
+                ("N", "C", "H", "W", "K", "kh", "kw", "sh", "sw", "pt", "pb", "pl", "pr")]
+
+    def out_hw(self):
+        return ((self.H + self.pt + self.pb - self.kh) // self.sh + 1,
+                (self.W + self.pl + self.pr - self.kw) // self.sw + 1)
+
+    def flops(self):
+        oh, ow = self.out_hw()
+        return 2.0 * self.N * self.K * self.C * oh * ow * self.kh * self.kw
+
+
+class GemmConfig(C.Structure):
+    _fields_ = [(n, C.c_int) for n in
+                ("id", "bm", "bn", "bk", "waves_m", "waves_n", "lds_bytes", "direct_lds")]
+
+
+class WinoPlan(C.Structure):
+    _fields_ = [("shape", ConvShape), ("OH", C.c_int), ("OW", C.c_int), ("tiles_h", C.c_int),
+                ("tiles_w", C.c_int), ("T", C.c_long), ("K_pad", C.c_int), ("C_pad", C.c_int),
+                ("T_pad", C.c_long), ("gemm_config", C.c_int), ("U_bytes", C.c_size_t),
+                ("V_bytes", C.c_size_t), ("M_bytes", C.c_size_t)]
+
+
+class IgemmPlan(C.Structure):
+    _fields_ = [("shape", ConvShape), ("OH", C.c_int), ("OW", C.c_int), ("Kred", C.c_int),
+                ("Kred_pad", C.c_int), ("K_pad", C.c_int), ("Npix", C.c_long), ("config", C.c_int),
+                ("Wp_bytes", C.c_size_t), ("table_bytes", C.c_size_t)]
+
+
+class DeviceInfo(C.Structure):
+    _fields_ = [("name", C.c_char * 128), ("arch", C.c_char * 32), ("compute_units", C.c_int),
+                ("clock_mhz", C.c_int), ("mem_clock_mhz", C.c_int), ("mem_bus_bits", C.c_int),
+                ("total_mem", C.c_size_t), ("lds_per_block", C.c_int)]
+
+
+# every symbol include/fastconv_hip.h declares: name -> (restype, argtypes)
+_vp = C.c_void_p
+_ABI = {
+    "fc_init": (C.c_int, [C.c_int, C.POINTER(_vp)]),
+    "fc_destroy": (C.c_int, [_vp]),
+    "fc_get_device_info": (C.c_int, [_vp, C.POINTER(DeviceInfo)]),
+    "fc_last_error": (C.c_char_p, [_vp]),
+    "fc_status_string": (C.c_char_p, [C.c_int]),
+    "fc_sync": (C.c_int, [_vp]),
+    "fc_pool_create": (C.c_int, [_vp, C.c_size_t, C.POINTER(_vp)]),
+    "fc_pool_destroy": (C.c_int, [_vp]),
+    "fc_pool_alloc": (C.c_int, [_vp, C.c_size_t, C.POINTER(_vp)]),
+    "fc_pool_reset": (C.c_int, [_vp]),
+    "fc_pool_mark": (C.c_int, [_vp, C.POINTER(C.c_size_t)]),
+    "fc_pool_release": (C.c_int, [_vp, C.c_size_t]),
+    "fc_pool_stats": (C.c_int, [_vp, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "fc_upload": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
+    "fc_download": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
+    "fc_fill_zero": (C.c_int, [_vp, _vp, C.c_size_t]),
+    "fc_timing_enable": (C.c_int, [_vp, C.c_int]),
+    "fc_timing_reset": (C.c_int, [_vp]),
+    "fc_stage_time_ms": (C.c_int, [_vp, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_long)]),
+    "fc_wino_gemm_num_configs": (C.c_int, []),
+    "fc_wino_gemm_get_config": (C.c_int, [C.c_int, C.POINTER(GemmConfig)]),
+    "fc_wino_make_plan": (C.c_int, [C.POINTER(ConvShape), C.c_int, C.POINTER(WinoPlan)]),
+    "fc_wino_filter_transform": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp]),
+    "fc_wino_input_transform": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp]),
+    "fc_wino_gemm": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, _vp]),
+    "fc_wino_output_transform": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, C.c_int, _vp]),
+    "fc_wino_forward": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, _vp, C.c_int, C.c_int,
+                                  _vp, _vp, _vp, _vp]),
+    "fc_igemm_num_configs": (C.c_int, []),
+    "fc_igemm_get_config": (C.c_int, [C.c_int, C.POINTER(GemmConfig)]),
+    "fc_igemm_make_plan": (C.c_int, [C.POINTER(ConvShape), C.c_int, C.POINTER(IgemmPlan)]),
+    "fc_igemm_pack_filter": (C.c_int, [_vp, C.POINTER(IgemmPlan), _vp, _vp, _vp]),
+    "fc_conv_implicit_gemm": (C.c_int, [_vp, C.POINTER(IgemmPlan), _vp, _vp, _vp, _vp, C.c_int, _vp]),
+}
+
+
+def abi_symbols():
+    return sorted(_ABI)
+
+
+def build_native(force=True):
+    """Compile the HIP library (and the C++ host driver) for gfx950."""
+    cmd = ["make", "-C", _HERE, "-j8", "all"]
+    if force:
+        cmd.insert(3, "-B")
+    subprocess.check_call(cmd)
+
+
+def load_cdll():
+    if not os.path.exists(LIB_PATH):
+        raise FastConvError(-2, "native library %s is missing: run __graft_entry__.build() "
+                            "(there is no CPU fallback)" % LIB_PATH)
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in _ABI.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+class Library:
+    """One context + one arena on one GPU; thin, typed wrappers over the C ABI."""
+
+    def __init__(self, device=0, pool_bytes=1 << 30):
+        self.c = load_cdll()
+        self.ctx = _vp()
+        rc = self.c.fc_init(device, C.byref(self.ctx))
+        if rc:
+            raise FastConvError(rc, self.c.fc_status_string(rc).decode())
+        self.pool = _vp()
+        self._check(self.c.fc_pool_create(self.ctx, pool_bytes, C.byref(self.pool)))
+
+    def close(self):
+        if self.pool:
+            self.c.fc_pool_destroy(self.pool)
+            self.pool = None
+        if self.ctx:
+            self.c.fc_destroy(self.ctx)
+            self.ctx = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def _check(self, rc):
+        if rc:
+            raise FastConvError(rc, self.c.fc_last_error(self.ctx).decode())
+
+    # ---- memory
+    def alloc(self, nbytes):
+        p = _vp()
+        self._check(self.c.fc_pool_alloc(self.pool, nbytes, C.byref(p)))
+        return p
+
+    def reset_pool(self):
+        self._check(self.c.fc_pool_reset(self.pool))
+
+    def pool_stats(self):
+        a, b, c_ = C.c_size_t(), C.c_size_t(), C.c_size_t()
+        self._check(self.c.fc_pool_stats(self.pool, C.byref(a), C.byref(b), C.byref(c_)))
+        return a.value, b.value, c_.value
+
+    def upload(self, arr):
+        arr = np.ascontiguousarray(arr)
+        p = self.alloc(max(arr.nbytes, 4))
+        self._check(self.c.fc_upload(self.ctx, p, arr.ctypes.data_as(_vp), arr.nbytes))
+        return p
+
+    def download(self, ptr, shape, dtype=np.float32):
+        out = np.empty(shape, dtype)
+        self._check(self.c.fc_download(self.ctx, out.ctypes.data_as(_vp), ptr, out.nbytes))
+        return out
+
+    def fill_zero(self, ptr, nbytes):
+        self._check(self.c.fc_fill_zero(self.ctx, ptr, nbytes))
+
+    def sync(self):
+        self._check(self.c.fc_sync(self.ctx))
+
+    def device_info(self):
+        info = DeviceInfo()
+        self._check(self.c.fc_get_device_info(self.ctx, C.byref(info)))
+        return {"name": info.name.decode(), "arch": info.arch.decode(), "compute_units": info.compute_units,
+                "clock_mhz": info.clock_mhz, "mem_clock_mhz": info.mem_clock_mhz,
+                "mem_bus_bits": info.mem_bus_bits, "total_mem": info.total_mem,
+                "lds_per_block": info.lds_per_block}
+
+    # ---- timing
+    def timing(self, on):
+        self._check(self.c.fc_timing_enable(self.ctx, 1 if on else 0))
+
+    def timing_reset(self):
+        self._check(self.c.fc_timing_reset(self.ctx))
+
+    def stage_time(self, stage):
+        ms, cnt = C.c_double(), C.c_long()
+        self._check(self.c.fc_stage_time_ms(self.ctx, stage, C.byref(ms), C.byref(cnt)))
+        return ms.value, cnt.value
+
+    # ---- configs / plans
+    def wino_configs(self):
+        out = []
+        for i in range(self.c.fc_wino_gemm_num_configs()):
+            g = GemmConfig()
+            self.c.fc_wino_gemm_get_config(i, C.byref(g))
+            out.append(g)
+        return out
+
+    def igemm_configs(self):
+        out = []
+        for i in range(self.c.fc_igemm_num_configs()):
+            g = GemmConfig()
+            self.c.fc_igemm_get_config(i, C.byref(g))
+            out.append(g)
+        return out
+
+    def wino_plan(self, shape, config=0):
+        plan = WinoPlan()
+        rc = self.c.fc_wino_make_plan(C.byref(shape), config, C.byref(plan))
+        if rc:
+            raise FastConvError(rc, self.c.fc_status_string(rc).decode())
+        return plan
+
+    def igemm_plan(self, shape, config=0):
+        plan = IgemmPlan()
+        rc = self.c.fc_igemm_make_plan(C.byref(shape), config, C.byref(plan))
+        if rc:
+            raise FastConvError(rc, self.c.fc_status_string(rc).decode())
+        return plan
+
+    # ---- Winograd stages
+    def wino_filter_transform(self, plan, w, U):
+        self._check(self.c.fc_wino_filter_transform(self.ctx, C.byref(plan), w, U))
+
+    def wino_input_transform(self, plan, x, V):
+        self._check(self.c.fc_wino_input_transform(self.ctx, C.byref(plan), x, V))
+
+    def wino_gemm(self, plan, U, V, M):
+        self._check(self.c.fc_wino_gemm(self.ctx, C.byref(plan), U, V, M))
+
+    def wino_output_transform(self, plan, M, y, bias=None, relu=False):
+        self._check(self.c.fc_wino_output_transform(self.ctx, C.byref(plan), M, bias, int(relu), y))
+
+    def wino_forward(self, plan, x, w, U, V, M, y, bias=None, relu=False, filter_ready=False):
+        self._check(self.c.fc_wino_forward(self.ctx, C.byref(plan), x, w, bias, int(relu),
+                                           int(filter_ready), U, V, M, y))
+
+    # ---- implicit GEMM
+    def igemm_pack_filter(self, plan, w, Wp, table):
+        self._check(self.c.fc_igemm_pack_filter(self.ctx, C.byref(plan), w, Wp, table))
+
+    def conv_implicit_gemm(self, plan, x, Wp, table, y, bias=None, relu=False):
+        self._check(self.c.fc_conv_implicit_gemm(self.ctx, C.byref(plan), x, Wp, table, bias, int(relu), y))
+
+    # ---- whole-layer helpers over host arrays (tests, smoke)
+    def winograd_conv(self, shape, x, w, bias=None, relu=False, config=0, stages=False):
+        plan = self.wino_plan(shape, config)
+        mark = C.c_size_t()
+        self._check(self.c.fc_pool_mark(self.pool, C.byref(mark)))
+        try:
+            dx, dw = self.upload(x), self.upload(w)
+            db = self.upload(bias) if bias is not None else None
+            U, V, M = self.alloc(plan.U_bytes), self.alloc(plan.V_bytes), self.alloc(plan.M_bytes)
+            y = self.alloc(4 * shape.N * shape.K * plan.OH * plan.OW)
+            self.wino_forward(plan, dx, dw, U, V, M, y, db, relu)
+            out = self.download(y, (shape.N, shape.K, plan.OH, plan.OW))
+            if not stages:
+                return out
+            Uh = self.download(U, (64, plan.C_pad, plan.K_pad))
+            Vh = self.download(V, (64, plan.C_pad, plan.T_pad))
+            Mh = self.download(M, (64, plan.K_pad, plan.T_pad))
+            return out, Uh, Vh, Mh, plan
+        finally:
+            self._check(self.c.fc_pool_release(self.pool, mark.value))
+
+    def implicit_gemm_conv(self, shape, x, w, bias=None, relu=False, config=0):
+        plan = self.igemm_plan(shape, config)
+        mark = C.c_size_t()
+        self._check(self.c.fc_pool_mark(self.pool, C.byref(mark)))
+        try:
+            dx, dw = self.upload(x), self.upload(w)
+            db = self.upload(bias) if bias is not None else None
+            Wp, tab = self.alloc(plan.Wp_bytes), self.alloc(plan.table_bytes)
+            y = self.alloc(4 * shape.N * shape.K * plan.OH * plan.OW)
+            self.igemm_pack_filter(plan, dw, Wp, tab)
+            self.conv_implicit_gemm(plan, dx, Wp, tab, y, db, relu)
+            return self.download(y, (shape.N, shape.K, plan.OH, plan.OW))
+        finally:
+            self._check(self.c.fc_pool_release(self.pool, mark.value))
+
+
+def load(device=0, pool_bytes=1 << 30):
+    return Library(device, pool_bytes)

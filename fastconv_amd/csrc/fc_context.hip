@@ -1,0 +1,298 @@
+// Context, memory arena, host<->device copies and stage timing of
+// libfastconv_hip.  No compute lives here.
+#include <cstdio>
+#include <cstring>
+#include <new>
+
+#include "fc_internal.h"
+
+int fc_set_error(fc_context *ctx, int status, const char *what, hipError_t err) {
+    if (ctx) {
+        char buf[512];
+        if (err != hipSuccess)
+            snprintf(buf, sizeof buf, "%s: %s (%s)", fc_status_string(status), what, hipGetErrorString(err));
+        else
+            snprintf(buf, sizeof buf, "%s: %s", fc_status_string(status), what);
+        ctx->last_error = buf;
+    }
+    return status;
+}
+
+bool fc_ctx_ok(const fc_context *ctx) { return ctx && ctx->magic == FC_CTX_MAGIC; }
+
+extern "C" const char *fc_status_string(int status) {
+    switch (status) {
+        case FC_OK: return "ok";
+        case FC_ERR_INVALID: return "invalid argument";
+        case FC_ERR_NO_DEVICE: return "no usable GPU";
+        case FC_ERR_HIP: return "HIP runtime error";
+        case FC_ERR_OOM: return "out of device memory";
+        case FC_ERR_STATE: return "wrong call order";
+        case FC_ERR_UNSUPPORTED: return "size not supported";
+        default: return "unknown status";
+    }
+}
+
+extern "C" int fc_init(int device, fc_context **out) {
+    if (!out) return FC_ERR_INVALID;
+    *out = nullptr;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0) {
+        (void)hipGetLastError();
+        return FC_ERR_NO_DEVICE;
+    }
+    if (device < 0 || device >= count) return FC_ERR_INVALID;
+    if (hipSetDevice(device) != hipSuccess) return FC_ERR_NO_DEVICE;
+    fc_context *ctx = new (std::nothrow) fc_context();
+    if (!ctx) return FC_ERR_OOM;
+    ctx->magic = FC_CTX_MAGIC;
+    ctx->device = device;
+    ctx->timing = false;
+    ctx->stream = nullptr;
+    memset(ctx->stage_ms, 0, sizeof ctx->stage_ms);
+    memset(ctx->stage_launches, 0, sizeof ctx->stage_launches);
+    if (hipGetDeviceProperties(&ctx->props, device) != hipSuccess) { delete ctx; return FC_ERR_NO_DEVICE; }
+    if (strncmp(ctx->props.gcnArchName, "gfx950", 6) != 0) {
+        fprintf(stderr, "fastconv: device %d is %s; this library holds gfx950 code only\n", device,
+                ctx->props.gcnArchName);
+        delete ctx;
+        return FC_ERR_NO_DEVICE;
+    }
+    if (hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking) != hipSuccess) { delete ctx; return FC_ERR_HIP; }
+    *out = ctx;
+    return FC_OK;
+}
+
+extern "C" int fc_destroy(fc_context *ctx) {
+    if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    for (auto &p : ctx->pending) { (void)hipEventDestroy(p.start); (void)hipEventDestroy(p.stop); }
+    for (auto &ev : ctx->free_events) (void)hipEventDestroy(ev);
+    (void)hipStreamDestroy(ctx->stream);
+    ctx->magic = 0;
+    delete ctx;
+    return FC_OK;
+}
+
+extern "C" int fc_get_device_info(fc_context *ctx, fc_device_info *info) {
+    if (!fc_ctx_ok(ctx) || !info) return FC_ERR_INVALID;
+    memset(info, 0, sizeof *info);
+    snprintf(info->name, sizeof info->name, "%s", ctx->props.name);
+    snprintf(info->arch, sizeof info->arch, "%s", ctx->props.gcnArchName);
+    info->compute_units = ctx->props.multiProcessorCount;
+    info->clock_mhz = ctx->props.clockRate / 1000;
+    info->mem_clock_mhz = ctx->props.memoryClockRate / 1000;
+    info->mem_bus_bits = ctx->props.memoryBusWidth;
+    info->total_mem = ctx->props.totalGlobalMem;
+    info->lds_per_block = (int)ctx->props.sharedMemPerBlock;
+    return FC_OK;
+}
+
+extern "C" const char *fc_last_error(fc_context *ctx) {
+    if (!fc_ctx_ok(ctx)) return "invalid context";
+    return ctx->last_error.c_str();
+}
+
+extern "C" int fc_sync(fc_context *ctx) {
+    if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    FC_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+    return FC_OK;
+}
+
+// ---------------------------------------------------------------- arena
+
+static const size_t kPoolAlign = 256;
+
+extern "C" int fc_pool_create(fc_context *ctx, size_t bytes, fc_pool **out) {
+    if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    if (!out || bytes == 0) return fc_set_error(ctx, FC_ERR_INVALID, "fc_pool_create: zero size or null out", hipSuccess);
+    *out = nullptr;
+    fc_pool *p = new (std::nothrow) fc_pool();
+    if (!p) return FC_ERR_OOM;
+    void *base = nullptr;
+    hipError_t e = hipMalloc(&base, bytes);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        delete p;
+        return fc_set_error(ctx, FC_ERR_OOM, "fc_pool_create: hipMalloc", e);
+    }
+    p->magic = FC_POOL_MAGIC;
+    p->ctx = ctx;
+    p->base = (char *)base;
+    p->capacity = bytes;
+    p->used = p->peak = 0;
+    *out = p;
+    return FC_OK;
+}
+
+extern "C" int fc_pool_destroy(fc_pool *pool) {
+    if (!pool || pool->magic != FC_POOL_MAGIC) return FC_ERR_STATE;
+    fc_context *ctx = pool->ctx;
+    if (fc_ctx_ok(ctx)) (void)hipStreamSynchronize(ctx->stream);
+    hipError_t e = hipFree(pool->base);
+    pool->magic = 0;
+    delete pool;
+    if (e != hipSuccess) return fc_set_error(ctx, FC_ERR_HIP, "fc_pool_destroy: hipFree", e);
+    return FC_OK;
+}
+
+extern "C" int fc_pool_alloc(fc_pool *pool, size_t bytes, void **dev_ptr) {
+    if (!pool || pool->magic != FC_POOL_MAGIC) return FC_ERR_STATE;
+    if (!dev_ptr) return FC_ERR_INVALID;
+    *dev_ptr = nullptr;
+    if (bytes == 0) return fc_set_error(pool->ctx, FC_ERR_INVALID, "fc_pool_alloc: zero bytes", hipSuccess);
+    const size_t start = (pool->used + kPoolAlign - 1) / kPoolAlign * kPoolAlign;
+    if (start > pool->capacity || bytes > pool->capacity - start) {
+        char msg[160];
+        snprintf(msg, sizeof msg, "fc_pool_alloc: %zu bytes requested, %zu of %zu in use", bytes, pool->used,
+                 pool->capacity);
+        return fc_set_error(pool->ctx, FC_ERR_OOM, msg, hipSuccess);
+    }
+    *dev_ptr = pool->base + start;
+    pool->used = start + bytes;
+    if (pool->used > pool->peak) pool->peak = pool->used;
+    return FC_OK;
+}
+
+extern "C" int fc_pool_reset(fc_pool *pool) {
+    if (!pool || pool->magic != FC_POOL_MAGIC) return FC_ERR_STATE;
+    pool->used = 0;
+    return FC_OK;
+}
+
+extern "C" int fc_pool_mark(fc_pool *pool, size_t *mark) {
+    if (!pool || pool->magic != FC_POOL_MAGIC) return FC_ERR_STATE;
+    if (!mark) return FC_ERR_INVALID;
+    *mark = pool->used;
+    return FC_OK;
+}
+
+extern "C" int fc_pool_release(fc_pool *pool, size_t mark) {
+    if (!pool || pool->magic != FC_POOL_MAGIC) return FC_ERR_STATE;
+    if (mark > pool->used) return fc_set_error(pool->ctx, FC_ERR_INVALID, "fc_pool_release: mark above current offset", hipSuccess);
+    pool->used = mark;
+    return FC_OK;
+}
+
+extern "C" int fc_pool_stats(fc_pool *pool, size_t *capacity, size_t *used, size_t *peak) {
+    if (!pool || pool->magic != FC_POOL_MAGIC) return FC_ERR_STATE;
+    if (capacity) *capacity = pool->capacity;
+    if (used) *used = pool->used;
+    if (peak) *peak = pool->peak;
+    return FC_OK;
+}
+
+// --------------------------------------------------------------- copies
+
+extern "C" int fc_upload(fc_context *ctx, void *dst_dev, const void *src_host, size_t bytes) {
+    if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    if (!dst_dev || !src_host) return fc_set_error(ctx, FC_ERR_INVALID, "fc_upload: null pointer", hipSuccess);
+    if (bytes == 0) return FC_OK;
+    FC_HIP_CHECK(ctx, hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream));
+    FC_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+    return FC_OK;
+}
+
+extern "C" int fc_download(fc_context *ctx, void *dst_host, const void *src_dev, size_t bytes) {
+    if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    if (!dst_host || !src_dev) return fc_set_error(ctx, FC_ERR_INVALID, "fc_download: null pointer", hipSuccess);
+    if (bytes == 0) return FC_OK;
+    FC_HIP_CHECK(ctx, hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    FC_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+    return FC_OK;
+}
+
+__global__ void fc_fill_zero_kernel(uint32_t *dst, size_t words) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < words; i += stride) dst[i] = 0u;
+}
+
+// A fill kernel rather than a memset node, so that callers may record it into a
+// HIP graph.
+extern "C" int fc_fill_zero(fc_context *ctx, void *dst_dev, size_t bytes) {
+    if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    if (!dst_dev || (bytes & 3) || ((uintptr_t)dst_dev & 3))
+        return fc_set_error(ctx, FC_ERR_INVALID, "fc_fill_zero: pointer and size must be 4-byte multiples", hipSuccess);
+    if (bytes == 0) return FC_OK;
+    const size_t words = bytes / 4;
+    size_t blocks = (words + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    fc_fill_zero_kernel<<<dim3((unsigned)blocks), dim3(256), 0, ctx->stream>>>((uint32_t *)dst_dev, words);
+    FC_LAUNCH_CHECK(ctx, "fc_fill_zero_kernel");
+    return FC_OK;
+}
+
+// --------------------------------------------------------------- timing
+
+static int fc_timing_fold(fc_context *ctx) {
+    if (ctx->pending.empty()) return FC_OK;
+    FC_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+    for (auto &p : ctx->pending) {
+        float ms = 0.f;
+        FC_HIP_CHECK(ctx, hipEventElapsedTime(&ms, p.start, p.stop));
+        ctx->stage_ms[p.stage] += ms;
+        ctx->stage_launches[p.stage] += 1;
+        ctx->free_events.push_back(p.start);
+        ctx->free_events.push_back(p.stop);
+    }
+    ctx->pending.clear();
+    return FC_OK;
+}
+
+static hipEvent_t fc_take_event(fc_context *ctx) {
+    if (!ctx->free_events.empty()) {
+        hipEvent_t ev = ctx->free_events.back();
+        ctx->free_events.pop_back();
+        return ev;
+    }
+    hipEvent_t ev = nullptr;
+    if (hipEventCreate(&ev) != hipSuccess) return nullptr;
+    return ev;
+}
+
+fc_stage_scope::fc_stage_scope(fc_context *c, int stage) : ctx(c), stop(nullptr), active(false) {
+    if (!c->timing) return;
+    if (c->pending.size() >= 8192) (void)fc_timing_fold(c);
+    hipEvent_t start = fc_take_event(c);
+    stop = fc_take_event(c);
+    if (!start || !stop) return;
+    (void)hipEventRecord(start, c->stream);
+    c->pending.push_back({stage, start, stop});
+    active = true;
+}
+
+fc_stage_scope::~fc_stage_scope() {
+    if (active) (void)hipEventRecord(stop, ctx->stream);
+}
+
+extern "C" int fc_timing_enable(fc_context *ctx, int on) {
+    if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    if (!on) {
+        const int rc = fc_timing_fold(ctx);
+        if (rc) return rc;
+    }
+    ctx->timing = on != 0;
+    return FC_OK;
+}
+
+extern "C" int fc_timing_reset(fc_context *ctx) {
+    if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    const int rc = fc_timing_fold(ctx);
+    if (rc) return rc;
+    memset(ctx->stage_ms, 0, sizeof ctx->stage_ms);
+    memset(ctx->stage_launches, 0, sizeof ctx->stage_launches);
+    return FC_OK;
+}
+
+extern "C" int fc_stage_time_ms(fc_context *ctx, int stage, double *total_ms, long *launches) {
+    if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    if (stage < 0 || stage >= FC_STAGE_COUNT) return fc_set_error(ctx, FC_ERR_INVALID, "fc_stage_time_ms: stage", hipSuccess);
+    const int rc = fc_timing_fold(ctx);
+    if (rc) return rc;
+    if (total_ms) *total_ms = ctx->stage_ms[stage];
+    if (launches) *launches = ctx->stage_launches[stage];
+    return FC_OK;
+}

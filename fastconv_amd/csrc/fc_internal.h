@@ -1,0 +1,99 @@
+// Internal declarations shared by the HIP translation units of libfastconv_hip.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <string>
+#include <vector>
+
+#include "fastconv_hip.h"
+
+struct fc_timing_pair {
+    int stage;
+    hipEvent_t start, stop;
+};
+
+struct fc_context {
+    uint32_t magic;
+    int device;
+    hipStream_t stream;
+    hipDeviceProp_t props;
+    std::string last_error;
+    bool timing;
+    std::vector<hipEvent_t> free_events;
+    std::vector<fc_timing_pair> pending;
+    double stage_ms[FC_STAGE_COUNT];
+    long stage_launches[FC_STAGE_COUNT];
+};
+
+struct fc_pool {
+    uint32_t magic;
+    fc_context *ctx;
+    char *base;
+    size_t capacity, used, peak;
+};
+
+static const uint32_t FC_CTX_MAGIC = 0x46434358u;   // "FCCX"
+static const uint32_t FC_POOL_MAGIC = 0x4643504cu;  // "FCPL"
+
+int fc_set_error(fc_context *ctx, int status, const char *what, hipError_t err);
+bool fc_ctx_ok(const fc_context *ctx);
+
+// Brackets one kernel launch with events when timing is on.
+struct fc_stage_scope {
+    fc_context *ctx;
+    hipEvent_t stop;
+    bool active;
+    fc_stage_scope(fc_context *c, int stage);
+    ~fc_stage_scope();
+};
+
+#define FC_HIP_CHECK(ctx, expr)                                              \
+    do {                                                                     \
+        hipError_t e__ = (expr);                                             \
+        if (e__ != hipSuccess) return fc_set_error((ctx), FC_ERR_HIP, #expr, e__); \
+    } while (0)
+
+#define FC_LAUNCH_CHECK(ctx, name)                                           \
+    do {                                                                     \
+        hipError_t e__ = hipGetLastError();                                  \
+        if (e__ != hipSuccess) return fc_set_error((ctx), FC_ERR_HIP, name, e__); \
+    } while (0)
+
+static inline long fc_round_up(long v, long m) { return (v + m - 1) / m * m; }
+
+static inline int fc_out_dim(int in, int pa, int pb, int k, int s) { return (in + pa + pb - k) / s + 1; }
+
+static inline bool fc_shape_ok(const fc_conv_shape *s) {
+    if (!s) return false;
+    if (s->N <= 0 || s->C <= 0 || s->H <= 0 || s->W <= 0 || s->K <= 0) return false;
+    if (s->kh <= 0 || s->kw <= 0 || s->sh <= 0 || s->sw <= 0) return false;
+    if (s->pt < 0 || s->pb < 0 || s->pl < 0 || s->pr < 0) return false;
+    if (s->H + s->pt + s->pb < s->kh || s->W + s->pl + s->pr < s->kw) return false;
+    return true;
+}
+
+// Unsigned division by a runtime constant: q = (n * mul) >> (32 + shift), exact
+// for n < 2^31 (round-up method with a 33-bit multiplier folded by one add).
+struct fc_fastdiv {
+    uint32_t mul, shift, div;
+};
+
+static inline fc_fastdiv fc_make_fastdiv(uint32_t d) {
+    fc_fastdiv f;
+    f.div = d;
+    if (d == 1) { f.mul = 0; f.shift = 0; return f; }
+    uint32_t l = 0;
+    while ((1ull << l) < d) l++;
+    // magic = ceil(2^(32+l) / d) - 2^32, fits 32 bits
+    const uint64_t m = ((1ull << 32) * ((1ull << l) - d)) / d + 1;
+    f.mul = (uint32_t)m;
+    f.shift = l;
+    return f;
+}
+
+__device__ __forceinline__ uint32_t fc_div(uint32_t n, const fc_fastdiv f) {
+    if (f.div == 1) return n;
+    const uint32_t t = __umulhi(n, f.mul);
+    return (t + ((n - t) >> 1)) >> (f.shift - 1);
+}

@@ -1,0 +1,302 @@
+// Implicit-GEMM convolution on gfx950 fp32 MFMA:
+//   y[n][k][oh][ow] = sum_{c,r,s} w[k][c][r][s] * x[n][c][oh*sh + r - pt][ow*sw + s - pl]
+// seen as D[K][N*OH*OW] = Wp^T[K][Kred] * col[Kred][N*OH*OW], where the column
+// matrix is never written to memory: each workgroup gathers its BK x BN slice of
+// it straight into LDS.  The filter is re-laid once to Wp[Kred_pad][K_pad]
+// (output channel fastest) so that its tiles are straight 16-byte copies, as in
+// the Winograd GEMM.
+#include "fc_internal.h"
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+// Row table entry for reduction index kred = (c*kh + r)*kw + s:
+//   [2*kred]   = c*H*W + r*W + s      (offset from the window origin)
+//   [2*kred+1] = r << 16 | s          (0x7fff7fff for padding rows: never in bounds)
+__global__ __launch_bounds__(256) void igemm_pack_filter_kernel(const float *__restrict__ w,
+                                                                float *__restrict__ Wp,
+                                                                int32_t *__restrict__ table, int K, int C,
+                                                                int kh, int kw, int H, int W, int Kred,
+                                                                int Kred_pad, int K_pad) {
+    const int k = blockIdx.x * 64 + (threadIdx.x & 63);
+    const int kred = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (kred >= Kred_pad) return;
+    if (k < K_pad) Wp[(size_t)kred * K_pad + k] = (k < K && kred < Kred) ? w[(size_t)k * Kred + kred] : 0.f;
+    if (blockIdx.x == 0 && (threadIdx.x & 63) == 0) {
+        if (kred < Kred) {
+            const int c = kred / (kh * kw), rs = kred - c * kh * kw, r = rs / kw, s = rs - r * kw;
+            table[2 * kred] = c * H * W + r * W + s;
+            table[2 * kred + 1] = (r << 16) | s;
+        } else {
+            table[2 * kred] = 0;
+            table[2 * kred + 1] = 0x7fff7fff;
+        }
+    }
+}
+
+struct IgemmParams {
+    const float *x;
+    const float *Wp;
+    const int32_t *table;
+    const float *bias;
+    float *y;
+    int N, C, H, W, K, OH, OW, sh, sw, pt, pl, relu;
+    int Kred_pad, K_pad;
+    long Npix;
+    int nKB, nPB;
+    fc_fastdiv divOHW, divOW;
+};
+
+template <int BM, int BN, int BK, int WGM, int WGN>
+struct IgTile {
+    static constexpr int BM_ = BM, BN_ = BN, BK_ = BK, WGM_ = WGM, WGN_ = WGN;
+    static constexpr int THREADS = 64 * WGM * WGN;
+    static constexpr int WM = BM / WGM, WN = BN / WGN;
+    static constexpr int MI = WM / 32, NI = WN / 32;
+    static constexpr int A_VEC = BK * BM / 4;
+    static constexpr int A_LD = (A_VEC + THREADS - 1) / THREADS;
+    static constexpr int ROW_STEP = THREADS / BN;       // gather: one column, every ROW_STEP-th row
+    static constexpr int B_LD = BK / ROW_STEP;
+    static constexpr int LDS_BYTES = 2 * BK * (BM + BN) * 4;
+    static_assert(THREADS % BN == 0 && BK % ROW_STEP == 0, "gather mapping");
+    static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be whole 32x32 MFMA blocks");
+};
+
+template <class TL>
+__global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmParams p) {
+    constexpr int BM = TL::BM_, BN = TL::BN_, BK = TL::BK_;
+    __shared__ __attribute__((aligned(16))) float As[2][BK][BM];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK][BN];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm0 = (wave / TL::WGN_) * TL::WM, wn0 = (wave % TL::WGN_) * TL::WN;
+    // output-channel blocks innermost: neighbouring workgroups share the gathered pixels
+    const int pb = blockIdx.x / p.nKB, kb = blockIdx.x - pb * p.nKB;
+
+    const float *Ag = p.Wp + (size_t)kb * BM;
+
+    // the pixel column this thread gathers
+    const int gcol = tid % BN, grow0 = tid / BN;
+    const long pix = (long)pb * BN + gcol;
+    const bool pixOK = pix < p.Npix;
+    int ih0 = 0, iw0 = 0;
+    const float *xwin = p.x;
+    if (pixOK) {
+        const uint32_t n = fc_div((uint32_t)pix, p.divOHW);
+        const uint32_t pp = (uint32_t)pix - n * (uint32_t)(p.OH * p.OW);
+        const uint32_t oh = fc_div(pp, p.divOW), ow = pp - oh * p.OW;
+        ih0 = (int)oh * p.sh - p.pt;
+        iw0 = (int)ow * p.sw - p.pl;
+        xwin = p.x + (size_t)n * p.C * p.H * p.W + (long)ih0 * p.W + iw0;
+    }
+
+    float4 ra[TL::A_LD];
+    float rb[TL::B_LD];
+
+    auto load_global = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < TL::A_LD; i++) {
+            const int v = tid + i * TL::THREADS;
+            if (TL::A_VEC % TL::THREADS == 0 || v < TL::A_VEC) {
+                const int row = v / (BM / 4), col = (v % (BM / 4)) * 4;
+                ra[i] = *reinterpret_cast<const float4 *>(Ag + (size_t)(k0 + row) * p.K_pad + col);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < TL::B_LD; i++) {
+            const int kred = k0 + grow0 + i * TL::ROW_STEP;
+            const int off = p.table[2 * kred], rs = p.table[2 * kred + 1];
+            const int ih = ih0 + (rs >> 16), iw = iw0 + (rs & 0xffff);
+            const bool ok = pixOK && (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
+            rb[i] = ok ? xwin[off] : 0.f;
+        }
+    };
+    auto store_lds = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < TL::A_LD; i++) {
+            const int v = tid + i * TL::THREADS;
+            if (TL::A_VEC % TL::THREADS == 0 || v < TL::A_VEC) {
+                const int row = v / (BM / 4), col = (v % (BM / 4)) * 4;
+                *reinterpret_cast<float4 *>(&As[buf][row][col]) = ra[i];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < TL::B_LD; i++) Bs[buf][grow0 + i * TL::ROW_STEP][gcol] = rb[i];
+    };
+
+    floatx16 acc[TL::MI][TL::NI];
+#pragma unroll
+    for (int mi = 0; mi < TL::MI; mi++)
+#pragma unroll
+        for (int ni = 0; ni < TL::NI; ni++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[mi][ni][i] = 0.f;
+
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+
+    const int lrow = lane >> 5, lcol = lane & 31;
+    const int nStages = p.Kred_pad / BK;
+    for (int s = 0; s < nStages; s++) {
+        const int cur = s & 1;
+        if (s + 1 < nStages) load_global((s + 1) * BK);
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 2) {
+            float a[TL::MI], bb[TL::NI];
+#pragma unroll
+            for (int mi = 0; mi < TL::MI; mi++) a[mi] = As[cur][kk + lrow][wm0 + mi * 32 + lcol];
+#pragma unroll
+            for (int ni = 0; ni < TL::NI; ni++) bb[ni] = Bs[cur][kk + lrow][wn0 + ni * 32 + lcol];
+#pragma unroll
+            for (int mi = 0; mi < TL::MI; mi++)
+#pragma unroll
+                for (int ni = 0; ni < TL::NI; ni++)
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[mi], bb[ni], acc[mi][ni], 0, 0, 0);
+        }
+        if (s + 1 < nStages) store_lds(cur ^ 1);
+        __syncthreads();
+    }
+
+    // epilogue: column = pixel (lane%32), rows = output channels
+    const int OHW = p.OH * p.OW;
+#pragma unroll
+    for (int ni = 0; ni < TL::NI; ni++) {
+        const long opix = (long)pb * BN + wn0 + ni * 32 + lcol;
+        if (opix >= p.Npix) continue;
+        const uint32_t n = fc_div((uint32_t)opix, p.divOHW);
+        const uint32_t pp = (uint32_t)opix - n * (uint32_t)OHW;
+        float *yn = p.y + (size_t)n * p.K * OHW + pp;
+#pragma unroll
+        for (int mi = 0; mi < TL::MI; mi++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int k = kb * BM + wm0 + mi * 32 + 8 * (i / 4) + 4 * lrow + (i % 4);
+                if (k < p.K) {
+                    float v = acc[mi][ni][i];
+                    if (p.bias) v += p.bias[k];
+                    if (p.relu) v = fmaxf(v, 0.f);
+                    yn[(size_t)k * OHW] = v;
+                }
+            }
+    }
+}
+
+typedef IgTile<128, 128, 16, 2, 2> Ig0;
+typedef IgTile<64, 128, 16, 1, 2> Ig1;
+typedef IgTile<128, 64, 16, 2, 1> Ig2;
+typedef IgTile<64, 64, 16, 2, 2> Ig3;
+typedef IgTile<32, 64, 16, 1, 1> Ig4;
+typedef IgTile<256, 128, 16, 2, 2> Ig5;
+typedef IgTile<128, 256, 16, 2, 2> Ig6;
+typedef IgTile<64, 256, 16, 1, 4> Ig7;
+
+const fc_gemm_config kIgConfigs[] = {
+#define FC_CFG(id, T) {id, T::BM_, T::BN_, T::BK_, T::WGM_, T::WGN_, T::LDS_BYTES, 0}
+    FC_CFG(0, Ig0), FC_CFG(1, Ig1), FC_CFG(2, Ig2), FC_CFG(3, Ig3),
+    FC_CFG(4, Ig4), FC_CFG(5, Ig5), FC_CFG(6, Ig6), FC_CFG(7, Ig7),
+#undef FC_CFG
+};
+const int kNumIgConfigs = sizeof(kIgConfigs) / sizeof(kIgConfigs[0]);
+
+template <class TL>
+void launch(fc_context *ctx, IgemmParams &p) {
+    const dim3 grid((unsigned)(p.nKB * p.nPB));
+    igemm_conv_kernel<TL><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
+}
+
+}  // namespace
+
+extern "C" int fc_igemm_num_configs(void) { return kNumIgConfigs; }
+
+extern "C" int fc_igemm_get_config(int id, fc_gemm_config *cfg) {
+    if (!cfg || id < 0 || id >= kNumIgConfigs) return FC_ERR_INVALID;
+    *cfg = kIgConfigs[id];
+    return FC_OK;
+}
+
+extern "C" int fc_igemm_make_plan(const fc_conv_shape *s, int config, fc_igemm_plan *plan) {
+    if (!plan || !fc_shape_ok(s)) return FC_ERR_INVALID;
+    fc_gemm_config cfg;
+    const int rc = fc_igemm_get_config(config, &cfg);
+    if (rc) return rc;
+    if (s->kh > 0x7ffe || s->kw > 0x7ffe) return FC_ERR_UNSUPPORTED;
+    plan->shape = *s;
+    plan->OH = fc_out_dim(s->H, s->pt, s->pb, s->kh, s->sh);
+    plan->OW = fc_out_dim(s->W, s->pl, s->pr, s->kw, s->sw);
+    const long kred = (long)s->C * s->kh * s->kw;
+    const long npix = (long)s->N * plan->OH * plan->OW;
+    if (kred >= (1l << 28) || npix >= (1l << 31) || (long)s->C * s->H * s->W >= (1l << 31)) return FC_ERR_UNSUPPORTED;
+    plan->Kred = (int)kred;
+    plan->Kred_pad = (int)fc_round_up(kred, cfg.bk);
+    plan->K_pad = (int)fc_round_up(s->K, cfg.bm);
+    plan->Npix = npix;
+    plan->config = config;
+    plan->Wp_bytes = sizeof(float) * (size_t)plan->Kred_pad * plan->K_pad;
+    plan->table_bytes = sizeof(int32_t) * 2 * (size_t)plan->Kred_pad;
+    return FC_OK;
+}
+
+static int ig_plan_check(fc_context *ctx, const fc_igemm_plan *plan) {
+    if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    if (!plan) return fc_set_error(ctx, FC_ERR_INVALID, "null plan", hipSuccess);
+    fc_igemm_plan chk;
+    const int rc = fc_igemm_make_plan(&plan->shape, plan->config, &chk);
+    if (rc) return fc_set_error(ctx, rc, "plan does not describe a supported layer", hipSuccess);
+    if (chk.Kred_pad != plan->Kred_pad || chk.K_pad != plan->K_pad || chk.Npix != plan->Npix)
+        return fc_set_error(ctx, FC_ERR_INVALID, "plan fields were modified after fc_igemm_make_plan", hipSuccess);
+    return FC_OK;
+}
+
+extern "C" int fc_igemm_pack_filter(fc_context *ctx, const fc_igemm_plan *plan, const float *w_dev, float *Wp_dev,
+                                    int32_t *table_dev) {
+    const int rc = ig_plan_check(ctx, plan);
+    if (rc) return rc;
+    if (!w_dev || !Wp_dev || !table_dev) return fc_set_error(ctx, FC_ERR_INVALID, "fc_igemm_pack_filter: null buffer", hipSuccess);
+    const fc_conv_shape &s = plan->shape;
+    const dim3 grid((plan->K_pad + 63) / 64, (plan->Kred_pad + 3) / 4);
+    if (grid.y > 65535) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_igemm_pack_filter: reduction too long", hipSuccess);
+    fc_stage_scope scope(ctx, FC_STAGE_FILTER_PACK);
+    igemm_pack_filter_kernel<<<grid, dim3(256), 0, ctx->stream>>>(w_dev, Wp_dev, table_dev, s.K, s.C, s.kh, s.kw, s.H,
+                                                                 s.W, plan->Kred, plan->Kred_pad, plan->K_pad);
+    FC_LAUNCH_CHECK(ctx, "igemm_pack_filter_kernel");
+    return FC_OK;
+}
+
+extern "C" int fc_conv_implicit_gemm(fc_context *ctx, const fc_igemm_plan *plan, const float *x_dev,
+                                     const float *Wp_dev, const int32_t *table_dev, const float *bias_dev, int relu,
+                                     float *y_dev) {
+    const int rc = ig_plan_check(ctx, plan);
+    if (rc) return rc;
+    if (!x_dev || !Wp_dev || !table_dev || !y_dev)
+        return fc_set_error(ctx, FC_ERR_INVALID, "fc_conv_implicit_gemm: null buffer", hipSuccess);
+    if ((uintptr_t)Wp_dev & 15) return fc_set_error(ctx, FC_ERR_INVALID, "fc_conv_implicit_gemm: Wp must be 16-byte aligned", hipSuccess);
+    fc_gemm_config cfg;
+    fc_igemm_get_config(plan->config, &cfg);
+    const fc_conv_shape &s = plan->shape;
+    IgemmParams p;
+    p.x = x_dev; p.Wp = Wp_dev; p.table = table_dev; p.bias = bias_dev; p.y = y_dev;
+    p.N = s.N; p.C = s.C; p.H = s.H; p.W = s.W; p.K = s.K; p.OH = plan->OH; p.OW = plan->OW;
+    p.sh = s.sh; p.sw = s.sw; p.pt = s.pt; p.pl = s.pl; p.relu = relu;
+    p.Kred_pad = plan->Kred_pad; p.K_pad = plan->K_pad; p.Npix = plan->Npix;
+    p.nKB = plan->K_pad / cfg.bm;
+    p.nPB = (int)((plan->Npix + cfg.bn - 1) / cfg.bn);
+    p.divOHW = fc_make_fastdiv((uint32_t)(plan->OH * plan->OW));
+    p.divOW = fc_make_fastdiv((uint32_t)plan->OW);
+    if ((long)p.nKB * p.nPB >= (1l << 31)) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_conv_implicit_gemm: grid too large", hipSuccess);
+    fc_stage_scope scope(ctx, FC_STAGE_IMPLICIT_GEMM);
+    switch (plan->config) {
+        case 0: launch<Ig0>(ctx, p); break;
+        case 1: launch<Ig1>(ctx, p); break;
+        case 2: launch<Ig2>(ctx, p); break;
+        case 3: launch<Ig3>(ctx, p); break;
+        case 4: launch<Ig4>(ctx, p); break;
+        case 5: launch<Ig5>(ctx, p); break;
+        case 6: launch<Ig6>(ctx, p); break;
+        case 7: launch<Ig7>(ctx, p); break;
+        default: return fc_set_error(ctx, FC_ERR_INVALID, "fc_conv_implicit_gemm: unknown tile configuration", hipSuccess);
+    }
+    FC_LAUNCH_CHECK(ctx, "igemm_conv_kernel");
+    return FC_OK;
+}

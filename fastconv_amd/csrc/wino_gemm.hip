@@ -1,0 +1,215 @@
+// Batched fp32 GEMM of the Winograd pipeline on gfx950 MFMA:
+//   M[f][k][t] = sum_c U[f][c][k] * V[f][c][t]      f = 0..63, one launch.
+// Both operands are stored reduction-index-major with the GEMM row/column index
+// fastest, which is exactly the order v_mfma_f32_32x32x2_f32 wants its lanes in
+// (lane l holds row/col l%32 of reduction step l/32), so tiles go global -> LDS
+// as straight 16-byte copies and LDS -> registers as conflict-free dword reads.
+#include "fc_internal.h"
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+// Workgroup tile BM x BN x BK; WGM x WGN wavefronts, each owning
+// (BM/WGM) x (BN/WGN) of the tile as 32x32 MFMA blocks.
+template <int BM, int BN, int BK, int WGM, int WGN>
+struct GemmTile {
+    static constexpr int THREADS = 64 * WGM * WGN;
+    static constexpr int WM = BM / WGM, WN = BN / WGN;
+    static constexpr int MI = WM / 32, NI = WN / 32;
+    static constexpr int A_VEC = BK * BM / 4, B_VEC = BK * BN / 4;      // float4 per stage
+    static constexpr int A_LD = (A_VEC + THREADS - 1) / THREADS;
+    static constexpr int B_LD = (B_VEC + THREADS - 1) / THREADS;
+    static constexpr int LDS_BYTES = 2 * BK * (BM + BN) * 4;
+    static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be whole 32x32 MFMA blocks");
+    static_assert(BK % 2 == 0, "32x32x2 MFMA consumes two reduction steps");
+    static_assert(BM % 4 == 0 && BN % 4 == 0, "16-byte copies");
+};
+
+// Workgroups are dealt to the 8 XCDs round-robin by linear id.  All tiles of one
+// frequency share U[f] and re-read V[f] once per output-channel block, so a
+// frequency is kept on one XCD (one L2): linear id b -> xcd = b % 8, and the
+// b / 8 sequence walks that XCD's 8 frequencies one after another, output
+// channel blocks innermost.
+template <class TL>
+__global__ __launch_bounds__(TL::THREADS) void wino_gemm_kernel(const float *__restrict__ U,
+                                                                const float *__restrict__ V,
+                                                                float *__restrict__ M, int K_pad, int C_pad,
+                                                                int T_pad, int nKB, int nTB) {
+    constexpr int BM = TL::BM_, BN = TL::BN_, BK = TL::BK_;
+    __shared__ __attribute__((aligned(16))) float As[2][BK][BM];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK][BN];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm0 = (wave / TL::WGN_) * TL::WM, wn0 = (wave % TL::WGN_) * TL::WN;
+
+    const int b = blockIdx.x, xcd = b & 7, idx = b >> 3;
+    const int bpf = nKB * nTB;
+    const int fl = idx / bpf, rem = idx - fl * bpf;
+    const int f = fl * 8 + xcd;
+    const int tb = rem / nKB, kb = rem - tb * nKB;
+
+    const float *Ag = U + (size_t)f * C_pad * K_pad + (size_t)kb * BM;
+    const float *Bg = V + (size_t)f * C_pad * T_pad + (size_t)tb * BN;
+
+    float4 ra[TL::A_LD], rb[TL::B_LD];
+
+    auto load_global = [&](int c0) {
+#pragma unroll
+        for (int i = 0; i < TL::A_LD; i++) {
+            const int v = tid + i * TL::THREADS;
+            if (TL::A_VEC % TL::THREADS == 0 || v < TL::A_VEC) {
+                const int row = v / (BM / 4), col = (v % (BM / 4)) * 4;
+                ra[i] = *reinterpret_cast<const float4 *>(Ag + (size_t)(c0 + row) * K_pad + col);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < TL::B_LD; i++) {
+            const int v = tid + i * TL::THREADS;
+            if (TL::B_VEC % TL::THREADS == 0 || v < TL::B_VEC) {
+                const int row = v / (BN / 4), col = (v % (BN / 4)) * 4;
+                rb[i] = *reinterpret_cast<const float4 *>(Bg + (size_t)(c0 + row) * T_pad + col);
+            }
+        }
+    };
+    auto store_lds = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < TL::A_LD; i++) {
+            const int v = tid + i * TL::THREADS;
+            if (TL::A_VEC % TL::THREADS == 0 || v < TL::A_VEC) {
+                const int row = v / (BM / 4), col = (v % (BM / 4)) * 4;
+                *reinterpret_cast<float4 *>(&As[buf][row][col]) = ra[i];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < TL::B_LD; i++) {
+            const int v = tid + i * TL::THREADS;
+            if (TL::B_VEC % TL::THREADS == 0 || v < TL::B_VEC) {
+                const int row = v / (BN / 4), col = (v % (BN / 4)) * 4;
+                *reinterpret_cast<float4 *>(&Bs[buf][row][col]) = rb[i];
+            }
+        }
+    };
+
+    floatx16 acc[TL::MI][TL::NI];
+#pragma unroll
+    for (int mi = 0; mi < TL::MI; mi++)
+#pragma unroll
+        for (int ni = 0; ni < TL::NI; ni++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[mi][ni][i] = 0.f;
+
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+
+    const int lrow = lane >> 5, lcol = lane & 31;
+    const int nStages = C_pad / BK;
+    for (int s = 0; s < nStages; s++) {
+        const int cur = s & 1;
+        if (s + 1 < nStages) load_global((s + 1) * BK);
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 2) {
+            float a[TL::MI], bb[TL::NI];
+#pragma unroll
+            for (int mi = 0; mi < TL::MI; mi++) a[mi] = As[cur][kk + lrow][wm0 + mi * 32 + lcol];
+#pragma unroll
+            for (int ni = 0; ni < TL::NI; ni++) bb[ni] = Bs[cur][kk + lrow][wn0 + ni * 32 + lcol];
+#pragma unroll
+            for (int mi = 0; mi < TL::MI; mi++)
+#pragma unroll
+                for (int ni = 0; ni < TL::NI; ni++)
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[mi], bb[ni], acc[mi][ni], 0, 0, 0);
+        }
+        if (s + 1 < nStages) store_lds(cur ^ 1);
+        __syncthreads();
+    }
+
+    // D block layout: register i of lane l is row 8*(i/4) + 4*(l/32) + i%4, column l%32.
+    float *Mg = M + ((size_t)f * K_pad + (size_t)kb * BM + wm0) * T_pad + (size_t)tb * BN + wn0;
+#pragma unroll
+    for (int mi = 0; mi < TL::MI; mi++)
+#pragma unroll
+        for (int ni = 0; ni < TL::NI; ni++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int row = mi * 32 + 8 * (i / 4) + 4 * lrow + (i % 4);
+                Mg[(size_t)row * T_pad + ni * 32 + lcol] = acc[mi][ni][i];
+            }
+}
+
+template <int BM, int BN, int BK, int WGM, int WGN>
+struct TileCfg : GemmTile<BM, BN, BK, WGM, WGN> {
+    static constexpr int BM_ = BM, BN_ = BN, BK_ = BK, WGM_ = WGM, WGN_ = WGN;
+};
+
+typedef TileCfg<128, 128, 16, 2, 2> Cfg0;
+typedef TileCfg<64, 128, 16, 1, 2> Cfg1;
+typedef TileCfg<128, 64, 16, 2, 1> Cfg2;
+typedef TileCfg<64, 64, 16, 2, 2> Cfg3;
+typedef TileCfg<32, 32, 16, 1, 1> Cfg4;
+typedef TileCfg<128, 128, 8, 2, 2> Cfg5;
+typedef TileCfg<64, 128, 8, 1, 2> Cfg6;
+typedef TileCfg<256, 128, 16, 2, 2> Cfg7;
+typedef TileCfg<128, 256, 16, 2, 2> Cfg8;
+typedef TileCfg<128, 128, 32, 2, 2> Cfg9;
+typedef TileCfg<64, 32, 16, 2, 1> Cfg10;
+
+const fc_gemm_config kConfigs[] = {
+#define FC_CFG(id, T) {id, T::BM_, T::BN_, T::BK_, T::WGM_, T::WGN_, T::LDS_BYTES, 0}
+    FC_CFG(0, Cfg0), FC_CFG(1, Cfg1), FC_CFG(2, Cfg2), FC_CFG(3, Cfg3), FC_CFG(4, Cfg4), FC_CFG(5, Cfg5),
+    FC_CFG(6, Cfg6), FC_CFG(7, Cfg7), FC_CFG(8, Cfg8), FC_CFG(9, Cfg9), FC_CFG(10, Cfg10),
+#undef FC_CFG
+};
+const int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
+
+template <class TL>
+void launch(fc_context *ctx, const fc_wino_plan *plan, const float *U, const float *V, float *M) {
+    const int nKB = plan->K_pad / TL::BM_, nTB = (int)(plan->T_pad / TL::BN_);
+    const dim3 grid(64u * nKB * nTB);
+    wino_gemm_kernel<TL><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(U, V, M, plan->K_pad, plan->C_pad,
+                                                                      (int)plan->T_pad, nKB, nTB);
+}
+
+}  // namespace
+
+extern "C" int fc_wino_gemm_num_configs(void) { return kNumConfigs; }
+
+extern "C" int fc_wino_gemm_get_config(int id, fc_gemm_config *cfg) {
+    if (!cfg || id < 0 || id >= kNumConfigs) return FC_ERR_INVALID;
+    *cfg = kConfigs[id];
+    return FC_OK;
+}
+
+extern "C" int fc_wino_gemm(fc_context *ctx, const fc_wino_plan *plan, const float *U_dev, const float *V_dev,
+                            float *M_dev) {
+    if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    if (!plan || !U_dev || !V_dev || !M_dev) return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_gemm: null argument", hipSuccess);
+    fc_gemm_config cfg;
+    if (fc_wino_gemm_get_config(plan->gemm_config, &cfg)) return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_gemm: unknown tile configuration", hipSuccess);
+    // the kernel has no edge predication: the buffers must be padded to the tile
+    if (plan->K_pad <= 0 || plan->C_pad <= 0 || plan->T_pad <= 0 || plan->K_pad % cfg.bm || plan->C_pad % cfg.bk ||
+        plan->T_pad % cfg.bn)
+        return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_gemm: padded sizes are not multiples of the tile", hipSuccess);
+    const long blocks = 64l * (plan->K_pad / cfg.bm) * (plan->T_pad / cfg.bn);
+    if (blocks >= (1l << 31)) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_gemm: grid too large", hipSuccess);
+    if (((uintptr_t)U_dev | (uintptr_t)V_dev | (uintptr_t)M_dev) & 15)
+        return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_gemm: buffers must be 16-byte aligned", hipSuccess);
+    fc_stage_scope scope(ctx, FC_STAGE_TENSOR_GEMM);
+    switch (plan->gemm_config) {
+        case 0: launch<Cfg0>(ctx, plan, U_dev, V_dev, M_dev); break;
+        case 1: launch<Cfg1>(ctx, plan, U_dev, V_dev, M_dev); break;
+        case 2: launch<Cfg2>(ctx, plan, U_dev, V_dev, M_dev); break;
+        case 3: launch<Cfg3>(ctx, plan, U_dev, V_dev, M_dev); break;
+        case 4: launch<Cfg4>(ctx, plan, U_dev, V_dev, M_dev); break;
+        case 5: launch<Cfg5>(ctx, plan, U_dev, V_dev, M_dev); break;
+        case 6: launch<Cfg6>(ctx, plan, U_dev, V_dev, M_dev); break;
+        case 7: launch<Cfg7>(ctx, plan, U_dev, V_dev, M_dev); break;
+        case 8: launch<Cfg8>(ctx, plan, U_dev, V_dev, M_dev); break;
+        case 9: launch<Cfg9>(ctx, plan, U_dev, V_dev, M_dev); break;
+        case 10: launch<Cfg10>(ctx, plan, U_dev, V_dev, M_dev); break;
+        default: return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_gemm: unknown tile configuration", hipSuccess);
+    }
+    FC_LAUNCH_CHECK(ctx, "wino_gemm_kernel");
+    return FC_OK;
+}

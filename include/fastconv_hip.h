@@ -1,0 +1,216 @@
+/*
+ * fastconv_hip.h -- C ABI of the MI355X (gfx950) convolution kernels.
+ *
+ * This is the boundary the C++ host layers (ConvWinoF63ZCLayer, ConvWinoF63Layer,
+ * ConvIm2colLayer) call; it is also what any other binding (ctypes, cgo, JNI)
+ * would load.  Plain pointers and sizes only.  Every function returns 0
+ * (FC_OK) or a negative fc_status; nothing throws across the boundary.  A
+ * context owns one HIP stream; calls on one context are ordered on that stream
+ * and must come from one thread at a time.
+ *
+ * Each entry point names the reference interface it stands in for (paths
+ * relative to the reference checkout).
+ */
+#ifndef FASTCONV_HIP_H_
+#define FASTCONV_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    FC_OK = 0,
+    FC_ERR_INVALID = -1,      /* bad argument / unsupported shape for this entry point */
+    FC_ERR_NO_DEVICE = -2,    /* no usable gfx950 device */
+    FC_ERR_HIP = -3,          /* a HIP runtime call failed; see fc_last_error() */
+    FC_ERR_OOM = -4,          /* pool exhausted or hipMalloc failed */
+    FC_ERR_STATE = -5,        /* call made in the wrong order (e.g. after destroy) */
+    FC_ERR_UNSUPPORTED = -6   /* size beyond a stated limit of the kernel */
+} fc_status;
+
+typedef struct fc_context fc_context;
+typedef struct fc_pool fc_pool;
+
+/* Convolution geometry, fp32 NCHW, group 1.  Field meaning follows the
+ * ConvLayer constructor arguments (conv_layer.h:27) plus a batch count. */
+typedef struct {
+    int N, C, H, W;
+    int K, kh, kw;
+    int sh, sw;
+    int pt, pb, pl, pr;
+} fc_conv_shape;
+
+/* Stages whose device time can be read back, labelled as the reference prints
+ * them (convLayer/winoF63ConvZC.cpp:249-253, convLayer/im2colConv.cpp:254-256). */
+typedef enum {
+    FC_STAGE_KERNEL_TRAN = 0,
+    FC_STAGE_INPUT_TRAN = 1,
+    FC_STAGE_TENSOR_GEMM = 2,
+    FC_STAGE_OUTPUT_TRAN = 3,
+    FC_STAGE_IMPLICIT_GEMM = 4,
+    FC_STAGE_FILTER_PACK = 5,
+    FC_STAGE_FUSED_GEMM_OUT = 6,
+    FC_STAGE_COUNT = 7
+} fc_stage;
+
+typedef struct {
+    char name[128];
+    char arch[32];
+    int compute_units;
+    int clock_mhz;
+    int mem_clock_mhz;
+    int mem_bus_bits;
+    size_t total_mem;
+    int lds_per_block;
+} fc_device_info;
+
+/* ---- context ---------------------------------------------------------- */
+
+/* Replaces the implicit process-wide state of the reference (one process,
+ * OpenMP threads set in conv_layer.h:31).  Fails with FC_ERR_NO_DEVICE when no
+ * GPU is present: there is no CPU fallback. */
+int fc_init(int device, fc_context **out);
+int fc_destroy(fc_context *ctx);
+int fc_get_device_info(fc_context *ctx, fc_device_info *info);
+const char *fc_last_error(fc_context *ctx);
+const char *fc_status_string(int status);
+int fc_sync(fc_context *ctx);
+
+/* ---- memory: one hipMalloc'd arena ------------------------------------ */
+
+/* Stands in for the allocations behind CommonMemPool / PrivateMemPool
+ * (utility/mempool.h:23-71) and _mm_malloc (utility/common.cpp:26-40): one
+ * device allocation per pool, sub-allocated by bumping a 256-byte aligned
+ * offset.  fc_pool_reset() rewinds to empty; fc_pool_mark/release rewind to a
+ * saved offset (scratch that lives for one Tuning() candidate). */
+int fc_pool_create(fc_context *ctx, size_t bytes, fc_pool **out);
+int fc_pool_destroy(fc_pool *pool);
+int fc_pool_alloc(fc_pool *pool, size_t bytes, void **dev_ptr);
+int fc_pool_reset(fc_pool *pool);
+int fc_pool_mark(fc_pool *pool, size_t *mark);
+int fc_pool_release(fc_pool *pool, size_t mark);
+int fc_pool_stats(fc_pool *pool, size_t *capacity, size_t *used, size_t *peak);
+
+/* Stand in for the memcpy()s into the layer's own buffers (conv_layer.h:74-77). */
+int fc_upload(fc_context *ctx, void *dst_dev, const void *src_host, size_t bytes);
+int fc_download(fc_context *ctx, void *dst_host, const void *src_dev, size_t bytes);
+int fc_fill_zero(fc_context *ctx, void *dst_dev, size_t bytes);
+
+/* ---- stage timing (utility/helper.h:66-80 Timer, per stage) ----------- */
+
+/* When enabled, every kernel launch below is bracketed by two events on the
+ * context's stream.  fc_stage_time_ms() waits for the stream, folds the pending
+ * event pairs into per-stage totals and returns total milliseconds and launch
+ * count since the last fc_timing_reset(). */
+int fc_timing_enable(fc_context *ctx, int on);
+int fc_timing_reset(fc_context *ctx);
+int fc_stage_time_ms(fc_context *ctx, int stage, double *total_ms, long *launches);
+
+/* ---- Winograd F(6x6,3x3), stride 1 ------------------------------------ */
+
+/* Tile shapes of the batched GEMM stage.  The reference tunes
+ * ocBlock/tileBlock/icBlock and a 4x4 or 4x5 register kernel
+ * (convLayer/winoF63ConvZC.cpp:25-174); here a configuration is a workgroup
+ * tile BM (output channels) x BN (tiles) x BK (input channels) and a wave grid. */
+typedef struct {
+    int id;
+    int bm, bn, bk;
+    int waves_m, waves_n;
+    int lds_bytes;
+    int direct_lds;           /* 1: operands go global -> LDS without passing registers */
+} fc_gemm_config;
+
+int fc_wino_gemm_num_configs(void);
+int fc_wino_gemm_get_config(int id, fc_gemm_config *cfg);
+
+/* Buffer geometry for one layer under one GEMM configuration.  Frequencies
+ * f = 8*row + col of the transformed 8x8 tile; tiles t = (n*tiles_h + th)*tiles_w + tw.
+ *   U[64][C_pad][K_pad]   transformed filters, output channel fastest
+ *   V[64][C_pad][T_pad]   transformed input tiles, tile fastest
+ *   M[64][K_pad][T_pad]   per-frequency products, tile fastest
+ * Padding (to the GEMM tile) is written as zeros by the transforms.
+ * Stands in for the buffer sizing in ConvWinoF63ZCLayer::Init
+ * (convLayer/winoF63ConvZC.cpp:176-213). */
+typedef struct {
+    fc_conv_shape shape;
+    int OH, OW;
+    int tiles_h, tiles_w;
+    long T;
+    int K_pad, C_pad;
+    long T_pad;
+    int gemm_config;
+    size_t U_bytes, V_bytes, M_bytes;
+} fc_wino_plan;
+
+int fc_wino_make_plan(const fc_conv_shape *shape, int gemm_config, fc_wino_plan *plan);
+
+/* U = G g G^T.  Replaces the kernel transform inside winoF63_v1_single
+ * (winoF63ZC/winoF63ZC.cpp:433-500) and offline_kernel_transform_v1 (:242-322).
+ * w is K x C x 3 x 3. */
+int fc_wino_filter_transform(fc_context *ctx, const fc_wino_plan *plan,
+                             const float *w_dev, float *U_dev);
+
+/* V = B^T d B with zero-filled borders.  Replaces the input transform inside
+ * winoF63_v1_single (winoF63ZC/winoF63ZC.cpp:512-813). */
+int fc_wino_input_transform(fc_context *ctx, const fc_wino_plan *plan,
+                            const float *x_dev, float *V_dev);
+
+/* M[f] = U[f]^T-layout product over input channels for all 64 frequencies in
+ * one launch, on fp32 MFMA.  Replaces the depth x oc x tile loop nest calling
+ * TensorGEMMInnerKernel4x4x4_v3 (winoF63ZC/winoF63ZC.cpp:818-860,
+ * winoF63ZC/TensorGEMMZC.cpp:443-583).  M is overwritten, never accumulated. */
+int fc_wino_gemm(fc_context *ctx, const fc_wino_plan *plan,
+                 const float *U_dev, const float *V_dev, float *M_dev);
+
+/* Y = A^T m A clipped to the image, written NCHW, with an optional per-channel
+ * bias (K floats) and optional ReLU.  Replaces the output transform inside
+ * winoF63_v1_single (winoF63ZC/winoF63ZC.cpp:869-973). */
+int fc_wino_output_transform(fc_context *ctx, const fc_wino_plan *plan,
+                             const float *M_dev, const float *bias_dev, int relu,
+                             float *y_dev);
+
+/* All stages back to back: what winoF63_v1_single (winoF63ZC/winoF63ZC.h:5-6)
+ * does in one call.  filter_ready != 0 skips the filter transform (U already
+ * holds it: the "offline" strategy, ConvTest.cpp:230-243). */
+int fc_wino_forward(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev,
+                    const float *w_dev, const float *bias_dev, int relu, int filter_ready,
+                    float *U_dev, float *V_dev, float *M_dev, float *y_dev);
+
+/* ---- implicit GEMM (replaces im2col + pack + GEMM) -------------------- */
+
+int fc_igemm_num_configs(void);
+int fc_igemm_get_config(int id, fc_gemm_config *cfg);
+
+/* Filter re-layout done once at Init: Wp[Kred_pad][K_pad], output channel
+ * fastest, reduction index (c, r, s) as in the column matrix rows
+ * (convLayer/im2colConv.cpp:285-309); plus the per-row gather table. */
+typedef struct {
+    fc_conv_shape shape;
+    int OH, OW;
+    int Kred, Kred_pad, K_pad;
+    long Npix;
+    int config;
+    size_t Wp_bytes, table_bytes;
+} fc_igemm_plan;
+
+int fc_igemm_make_plan(const fc_conv_shape *shape, int config, fc_igemm_plan *plan);
+
+/* Replaces pack_a_v2 (im2col/gemm_pack.cpp:192-260) as a one-time step. */
+int fc_igemm_pack_filter(fc_context *ctx, const fc_igemm_plan *plan, const float *w_dev,
+                         float *Wp_dev, int32_t *table_dev);
+
+/* y[n][k][oh][ow] = sum_{c,r,s} w[k][c][r][s] * x[n][c][oh*sh+r-pt][ow*sw+s-pl].
+ * Replaces ConvIm2colLayer::im2col_v1 + sgemm (convLayer/im2colConv.cpp:311-398,
+ * 434-565) and the register kernels of im2col/gemm_kernel.cpp; the column matrix
+ * is never materialised and y is overwritten (not accumulated). */
+int fc_conv_implicit_gemm(fc_context *ctx, const fc_igemm_plan *plan, const float *x_dev,
+                          const float *Wp_dev, const int32_t *table_dev,
+                          const float *bias_dev, int relu, float *y_dev);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
