@@ -1,0 +1,80 @@
+"""The C-ABI library loads and exports exactly what include/fastconv_hip.h
+declares.  No compute is called here (this file runs without a GPU)."""
+import ctypes as C
+import os
+import re
+
+from fastconv_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "fastconv_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fc_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_name_the_same_symbols():
+    assert _declared() == capi.abi_symbols()
+
+
+def test_library_exports_every_declared_symbol():
+    lib = C.CDLL(capi.LIB_PATH)
+    for name in _declared():
+        assert hasattr(lib, name), name
+
+
+def test_status_strings_and_config_tables_need_no_gpu():
+    lib = capi.load_cdll()
+    assert lib.fc_status_string(0) == b"ok"
+    assert lib.fc_status_string(-4) == b"out of device memory"
+    n = lib.fc_wino_gemm_num_configs()
+    assert n >= 4
+    seen = set()
+    for i in range(n):
+        g = capi.GemmConfig()
+        assert lib.fc_wino_gemm_get_config(i, C.byref(g)) == 0
+        assert g.id == i and g.bm % 32 == 0 and g.bn % 32 == 0 and g.bk % 2 == 0
+        assert g.lds_bytes == 2 * g.bk * (g.bm + g.bn) * 4 <= 64 * 1024
+        seen.add((g.bm, g.bn, g.bk, g.waves_m, g.waves_n))
+    assert len(seen) == n
+    assert lib.fc_wino_gemm_get_config(n, C.byref(capi.GemmConfig())) == -1
+    for i in range(lib.fc_igemm_num_configs()):
+        g = capi.GemmConfig()
+        assert lib.fc_igemm_get_config(i, C.byref(g)) == 0
+        assert (64 * g.waves_m * g.waves_n) % g.bn == 0
+
+
+def test_plans_are_pure_host_arithmetic():
+    lib = capi.load_cdll()
+    s = capi.ConvShape(32, 256, 56, 56, 256, 3, 3, 1, 1, 1, 1, 1, 1)
+    p = capi.WinoPlan()
+    assert lib.fc_wino_make_plan(C.byref(s), 0, C.byref(p)) == 0
+    assert (p.OH, p.OW, p.tiles_h, p.tiles_w, p.T) == (56, 56, 10, 10, 3200)
+    assert (p.K_pad, p.C_pad, p.T_pad) == (256, 256, 3200)
+    assert p.V_bytes == 64 * 256 * 3200 * 4 and p.M_bytes == p.V_bytes and p.U_bytes == 64 * 256 * 256 * 4
+    # winoF63ZC/winoF63ZC.cpp:336-338: ceil(OH/6) tiles, also when OH is not a multiple of 6
+    s2 = capi.ConvShape(1, 3, 7, 9, 5, 3, 3, 1, 1, 1, 1, 1, 1)
+    assert lib.fc_wino_make_plan(C.byref(s2), 4, C.byref(p)) == 0
+    assert (p.tiles_h, p.tiles_w, p.T, p.K_pad, p.C_pad, p.T_pad) == (2, 2, 4, 32, 16, 32)
+    # Winograd is 3x3 stride 1 only
+    s3 = capi.ConvShape(1, 3, 8, 8, 5, 3, 3, 2, 2, 1, 1, 1, 1)
+    assert lib.fc_wino_make_plan(C.byref(s3), 0, C.byref(p)) == -1
+    q = capi.IgemmPlan()
+    assert lib.fc_igemm_make_plan(C.byref(s3), 0, C.byref(q)) == 0
+    assert (q.OH, q.OW, q.Kred, q.Npix) == (4, 4, 27, 16)
+    assert q.Kred_pad == 32 and q.K_pad == 128
+
+
+def test_no_gpu_means_a_loud_error_not_a_fallback():
+    import pytest
+    lib = capi.load_cdll()
+    ctx = C.c_void_p()
+    rc = lib.fc_init(0, C.byref(ctx))
+    if rc == 0:                       # a GPU is present: nothing to check here
+        lib.fc_destroy(ctx)
+        return
+    assert rc == -2 and not ctx.value
+    with pytest.raises(capi.FastConvError):
+        capi.Library(0)

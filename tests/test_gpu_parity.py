@@ -1,0 +1,264 @@
+"""Parity of the HIP kernels with the CPU oracle, through the C ABI, on a real
+MI355X.  Tolerances are the ones the workload definition states:
+  * implicit GEMM (im2col path):  max|y-ref| / max|ref| <= 1e-5
+  * Winograd F(6,3):              max|y-ref| / max|ref| <= 1e-3
+both against the fp64 direct convolution of the oracle on the same seeded
+inputs (the fp32 naive result is checked alongside).  Large shapes are covered
+by size-independent properties (delta/shift kernels, all-ones closed form,
+linearity, agreement of the two algorithms with each other).
+"""
+import os
+
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TOL_IM2COL = 1e-5
+TOL_WINO = 1e-3
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "naive_ref_vectors.npz")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    import fastconv_amd as F
+    L = F.load(0, 20 << 30)
+    yield L
+    L.close()
+
+
+def cshape(s):
+    import fastconv_amd as F
+    return F.ConvShape(*[getattr(s, n) for n, _ in F.ConvShape._fields_])
+
+
+def announce(*a):
+    print(*a, flush=True)
+
+
+# ------------------------------------------------------------ Winograd stages
+
+@pytest.mark.parametrize("shp,cfg", [
+    ((2, 3, 8, 11, 5), 4), ((1, 64, 56, 56, 64), 0), ((3, 10, 14, 14, 70), 3), ((1, 5, 30, 20, 33), 10),
+])
+def test_winograd_stage_by_stage(lib, shp, cfg):
+    s = O.shape(*shp)
+    x, w = O.make_inputs(s, seed=1)
+    announce("stages", shp, "cfg", cfg)
+    y, U, V, M, plan = lib.winograd_conv(cshape(s), x, w, config=cfg, stages=True)
+    Uo = O.wino_filter_transform(w)
+    Vo = O.wino_input_transform(s, x)
+    Mo = O.wino_gemm(Uo, Vo)
+    T = plan.T
+    # U[f][c][k] against the oracle's U[f][k][c]; padding is exact zeros
+    assert np.abs(U[:, :s.C, :s.K].transpose(0, 2, 1) - Uo).max() <= 1e-6 * np.abs(Uo).max()
+    assert not U[:, s.C:, :].any() and not U[:, :, s.K:].any()
+    assert np.abs(V[:, :s.C, :T] - Vo).max() <= 1e-5 * np.abs(Vo).max()
+    assert not V[:, s.C:, :].any() and not V[:, :, T:].any()
+    assert np.abs(M[:, :s.K, :T] - Mo).max() <= 1e-5 * np.abs(Mo).max()
+    assert not M[:, s.K:, :].any() and not M[:, :, T:].any()
+    assert O.max_rel_err(y, O.naive_conv_f64(s, x, w)) <= TOL_WINO
+
+
+# -------------------------------------------------------- Winograd whole conv
+
+WINO_SHAPES = [
+    (1, 64, 56, 56, 64),       # BASELINE config 1
+    (1, 1, 6, 6, 1), (1, 3, 7, 7, 7), (2, 64, 8, 8, 6), (1, 3, 13, 13, 5), (1, 64, 14, 14, 9),
+    (1, 1, 28, 28, 3), (1, 3, 56, 56, 2), (2, 5, 9, 23, 11), (1, 4, 224, 224, 3), (1, 2, 112, 112, 5),
+    (5, 7, 7, 7, 130), (32, 16, 14, 14, 16), (3, 130, 28, 28, 40),
+]
+
+
+@pytest.mark.parametrize("shp", WINO_SHAPES)
+def test_winograd_against_oracle(lib, shp):
+    s = O.shape(*shp)
+    x, w = O.make_inputs(s, seed=shp[1] * 7 + shp[2])
+    announce("winograd", shp)
+    y = lib.winograd_conv(cshape(s), x, w)
+    truth = O.naive_conv_f64(s, x, w)
+    assert O.max_rel_err(y, truth) <= TOL_WINO
+    assert O.max_rel_err(y, O.naive_conv_f32(s, x, w)) <= TOL_WINO
+    # and within fp32 rounding of the oracle's own Winograd restatement
+    assert O.max_rel_err(y, O.wino_conv_f32(s, x, w)) <= 1e-4
+
+
+def test_winograd_every_tile_config(lib):
+    s = O.shape(2, 40, 28, 28, 72)
+    x, w = O.make_inputs(s, seed=5)
+    truth = O.naive_conv_f64(s, x, w)
+    for cfg in lib.wino_configs():
+        announce("winograd tile config", cfg.id, cfg.bm, cfg.bn, cfg.bk)
+        y = lib.winograd_conv(cshape(s), x, w, config=cfg.id)
+        assert O.max_rel_err(y, truth) <= TOL_WINO, cfg.id
+
+
+@pytest.mark.parametrize("pad", [0, 2])
+def test_winograd_other_paddings(lib, pad):
+    s = O.shape(2, 6, 20, 17, 10, pt=pad)
+    x, w = O.make_inputs(s, seed=pad)
+    y = lib.winograd_conv(cshape(s), x, w)
+    assert y.shape == (2, 10) + O.out_hw(s)
+    assert O.max_rel_err(y, O.naive_conv_f64(s, x, w)) <= TOL_WINO
+
+
+def test_winograd_bias_relu_epilogue(lib):
+    s = O.shape(2, 8, 14, 14, 12)
+    x, w = O.make_inputs(s, seed=8)
+    bias = O.rng_uniform(3, (s.K,))
+    truth = np.maximum(O.naive_conv_f64(s, x, w, bias), 0.0)
+    y = lib.winograd_conv(cshape(s), x, w, bias=bias, relu=True)
+    assert (y >= 0).all()
+    assert O.max_rel_err(y, truth) <= TOL_WINO
+
+
+def test_winograd_rejects_unsupported(lib):
+    import fastconv_amd as F
+    for bad in [O.shape(1, 4, 8, 8, 4, 3, 3, 2, 2, 1), O.shape(1, 4, 8, 8, 4, 5, 5, 1, 1, 2),
+                O.shape(1, 4, 8, 8, 4, 1, 1, 1, 1, 0)]:
+        with pytest.raises(F.FastConvError):
+            lib.wino_plan(cshape(bad), 0)
+
+
+# -------------------------------------------------------------- implicit GEMM
+
+IGEMM_SHAPES = [
+    (1, 256, 56, 56, 256, 3, 3, 1, 1, 1),        # BASELINE config 2, layer A
+    (1, 128, 56, 56, 256, 3, 3, 2, 2, 1),        # layer B
+    (1, 256, 14, 14, 1024, 1, 1, 1, 1, 0),       # layer C
+    (1, 3, 224, 224, 64, 7, 7, 2, 2, 3),         # ResNet-50 stem
+    (1, 256, 56, 56, 128, 1, 1, 2, 2, 0),        # 1x1 stride-2 projection
+    (2, 2048, 7, 7, 512, 1, 1, 1, 1, 0),
+    (1, 1, 5, 5, 1, 3, 3, 1, 1, 1), (3, 5, 9, 8, 70, 3, 2, 2, 1, 1), (2, 7, 15, 15, 33, 5, 5, 3, 3, 2),
+]
+
+
+@pytest.mark.parametrize("shp", IGEMM_SHAPES)
+def test_implicit_gemm_against_oracle(lib, shp):
+    s = O.shape(*shp)
+    x, w = O.make_inputs(s, seed=shp[1] + shp[4])
+    announce("implicit gemm", shp)
+    y = lib.implicit_gemm_conv(cshape(s), x, w)
+    assert O.max_rel_err(y, O.naive_conv_f64(s, x, w)) <= TOL_IM2COL
+    assert O.max_rel_err(y, O.naive_conv_f32(s, x, w)) <= TOL_IM2COL
+
+
+def test_implicit_gemm_asymmetric_padding_and_bias(lib):
+    s = O.Shape(2, 4, 11, 12, 9, 5, 3, 1, 2, 0, 1, 2, 1)
+    x, w = O.make_inputs(s, seed=2)
+    bias = O.rng_uniform(4, (s.K,))
+    y = lib.implicit_gemm_conv(cshape(s), x, w, bias=bias, relu=True)
+    truth = np.maximum(O.naive_conv_f64(s, x, w, bias), 0.0)
+    assert O.max_rel_err(y, truth) <= TOL_IM2COL
+
+
+def test_implicit_gemm_every_tile_config(lib):
+    s = O.shape(2, 24, 19, 19, 72, 3, 3, 2, 2, 1)
+    x, w = O.make_inputs(s, seed=6)
+    truth = O.naive_conv_f64(s, x, w)
+    for cfg in lib.igemm_configs():
+        announce("implicit gemm tile config", cfg.id, cfg.bm, cfg.bn, cfg.bk)
+        y = lib.implicit_gemm_conv(cshape(s), x, w, config=cfg.id)
+        assert O.max_rel_err(y, truth) <= TOL_IM2COL, cfg.id
+
+
+# ------------------------------------------- the reference's own naive layers
+
+def test_golden_vectors_of_reference_naive_layers(lib):
+    z = np.load(GOLD)
+    names = sorted({k.split("/")[0] for k in z.files})
+    for name in names:
+        if name + "/bias_elems" in z.files:
+            continue                 # per-element bias tensor: not a fast-path feature
+        s = O.Shape(*[int(v) for v in z[name + "/shape"]])
+        x, w, y_ref = z[name + "/x"], z[name + "/w"], z[name + "/y"]
+        announce("golden", name)
+        y = lib.implicit_gemm_conv(cshape(s), x, w)
+        assert O.max_rel_err(y, y_ref) <= TOL_IM2COL, name
+        if s.kh == 3 and s.kw == 3 and s.sh == 1 and s.sw == 1:
+            yw = lib.winograd_conv(cshape(s), x, w)
+            assert O.max_rel_err(yw, y_ref) <= TOL_WINO, name
+
+
+# ------------------------------------------------ full-size layers: properties
+
+def _full_layers():
+    # (N, C, H, K): VGG-16 and ResNet-50 3x3 stride-1 layers at batch 32
+    return [(32, 3, 224, 64), (32, 64, 224, 64), (32, 128, 112, 128), (32, 256, 56, 256),
+            (32, 512, 28, 512), (32, 512, 14, 512), (32, 64, 56, 64), (32, 512, 7, 512)]
+
+
+@pytest.mark.parametrize("N,C,H,K", _full_layers())
+def test_full_size_shift_kernel_property(lib, N, C, H, K):
+    """With w[k][c] = delta(c == k % C) * one tap at (u, v), output channel k is
+    input channel k % C shifted by (u-1, v-1): an exact answer at any size."""
+    s = O.shape(N, C, H, H, K)
+    x = O.rng_uniform(11, (N, C, H, H))
+    u, v = 2, 0
+    w = np.zeros((K, C, 3, 3), np.float32)
+    w[np.arange(K), np.arange(K) % C, u, v] = 1.0
+    xp = np.pad(x, ((0, 0), (0, 0), (1, 1), (1, 1)))
+    expect = xp[:, np.arange(K) % C, u:u + H, v:v + H]
+    announce("full-size shift", (N, C, H, K))
+    yw = lib.winograd_conv(cshape(s), x, w)
+    assert O.max_rel_err(yw, expect) <= TOL_WINO
+    yi = lib.implicit_gemm_conv(cshape(s), x, w)
+    assert np.array_equal(yi, expect)            # one non-zero product per output: exact
+
+
+@pytest.mark.parametrize("N,C,H,K", [(32, 256, 56, 256), (32, 64, 224, 64), (32, 512, 14, 512)])
+def test_full_size_two_algorithms_agree_and_are_linear(lib, N, C, H, K):
+    s = O.shape(N, C, H, H, K)
+    x, w = O.make_inputs(s, seed=1)
+    announce("full-size agreement", (N, C, H, K))
+    yw = lib.winograd_conv(cshape(s), x, w)
+    yi = lib.implicit_gemm_conv(cshape(s), x, w)
+    assert O.max_rel_err(yw, yi) <= TOL_WINO
+    # spot-check 3 images' worth of output channels against the fp64 oracle
+    sub = O.shape(1, C, H, H, K)
+    truth = O.naive_conv_f64(sub, np.ascontiguousarray(x[N - 1:N]), w)
+    assert O.max_rel_err(yi[N - 1:N], truth) <= TOL_IM2COL
+    assert O.max_rel_err(yw[N - 1:N], truth) <= TOL_WINO
+    # linearity in the input: conv(2x) == 2 conv(x) exactly in binary floating point
+    y2 = lib.winograd_conv(cshape(s), 2.0 * x, w)
+    assert np.array_equal(y2, 2.0 * yw)
+
+
+def test_all_ones_closed_form_full_size(lib):
+    s = O.shape(32, 128, 112, 112, 128)
+    x = np.ones((s.N, s.C, s.H, s.W), np.float32)
+    w = np.ones((s.K, s.C, 3, 3), np.float32)
+    cnt = np.full((112, 112), 9.0)
+    cnt[0, :] = cnt[-1, :] = cnt[:, 0] = cnt[:, -1] = 6.0
+    cnt[0, 0] = cnt[0, -1] = cnt[-1, 0] = cnt[-1, -1] = 4.0
+    expect = np.broadcast_to(s.C * cnt, (s.N, s.K, 112, 112))
+    yi = lib.implicit_gemm_conv(cshape(s), x, w)
+    assert np.array_equal(yi, expect)
+    yw = lib.winograd_conv(cshape(s), x, w)
+    assert O.max_rel_err(yw, expect) <= TOL_WINO
+
+
+# ----------------------------------------------------------------- the arena
+
+def test_pool_exhaustion_is_reported(lib):
+    import fastconv_amd as F
+    cap, used, _ = lib.pool_stats()
+    with pytest.raises(F.FastConvError) as e:
+        lib.alloc(cap + 1)
+    assert e.value.status == -4
+    assert lib.pool_stats()[1] == used
+
+
+def test_stage_timers_count_launches(lib):
+    s = O.shape(1, 8, 12, 12, 8)
+    x, w = O.make_inputs(s)
+    lib.timing(True)
+    lib.timing_reset()
+    lib.winograd_conv(cshape(s), x, w)
+    lib.winograd_conv(cshape(s), x, w)
+    for stage in range(4):
+        ms, cnt = lib.stage_time(stage)
+        assert cnt == 2 and ms > 0.0
+    lib.timing(False)
