@@ -1,0 +1,280 @@
+#!/usr/bin/env python3
+"""Throughput of the convolution hot path on one MI355X.
+
+A "step" is one forward pass of every conv layer of the workload (default: the
+13 3x3 conv layers of VGG-16 at batch 32, Winograd F(6x6,3x3), filter transform
+included) over synthetic inputs already resident in HBM.  Prints ONE JSON line:
+whole-job effective GFLOP/s (direct-convolution FLOP count / wall time), the
+roofline of the dominant kernel (the batched Winograd GEMM, timed with HIP
+events on the library's stream inside the timed region), and a CPU baseline (the
+naive direct convolution on the host cores, on a bounded sample).
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_MFMA_F32_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+# (C, K, H, repeats)
+VGG16 = [(3, 64, 224, 1), (64, 64, 224, 1), (64, 128, 112, 1), (128, 128, 112, 1), (128, 256, 56, 1),
+         (256, 256, 56, 2), (256, 512, 28, 1), (512, 512, 28, 2), (512, 512, 14, 3)]
+RESNET50_3X3 = [(64, 64, 56, 3), (128, 128, 28, 4), (256, 256, 14, 6), (512, 512, 7, 3)]
+STRESS = [(256, 256, 56, 1), (512, 512, 28, 1), (512, 512, 14, 1)]
+
+WORKLOADS = {
+    # name: (layers, batch, description)
+    "vgg16_b32": (VGG16, 32, "VGG-16 conv stack, 13 layers, 3x3 s1 p1, Winograd F(6,3), batch 32"),
+    "vgg16_b1": (VGG16, 1, "VGG-16 conv stack, 13 layers, 3x3 s1 p1, Winograd F(6,3), batch 1"),
+    "resnet50_3x3_b32": (RESNET50_3X3, 32, "ResNet-50 3x3 s1 bottleneck convs, Winograd F(6,3), batch 32"),
+    "resnet50_3x3_b1": (RESNET50_3X3, 1, "ResNet-50 3x3 s1 bottleneck convs, Winograd F(6,3), batch 1"),
+    "cfg1": ([(64, 64, 56, 1)], 1, "single 3x3 conv 64->64 @56, batch 1"),
+    "stress_b64": (STRESS, 64, "VGG-16 256@56, 512@28, 512@14, batch 64"),
+    "stress_b128": (STRESS, 128, "VGG-16 256@56, 512@28, 512@14, batch 128"),
+}
+
+ST_KT, ST_IT, ST_GEMM, ST_OT = 0, 1, 2, 3
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+class Layer:
+    """One conv layer with its buffers resident on the device."""
+
+    def __init__(self, L, F, N, C, K, H, repeats, rng):
+        self.N, self.C, self.K, self.H, self.repeats = N, C, K, H, repeats
+        self.shape = F.ConvShape(N, C, H, H, K, 3, 3, 1, 1, 1, 1, 1, 1)
+        x = rng.random((N, C, H, H), dtype=np.float32) * 2.0 - 1.0
+        w = (rng.standard_normal((K, C, 3, 3), dtype=np.float32) * np.float32(np.sqrt(2.0 / (9 * C))))
+        self.x, self.w = L.upload(x), L.upload(w)
+        self.y = L.alloc(4 * N * K * H * H)
+        self.flops = self.shape.flops()
+        self.plan = None
+        self.U = None
+
+    def algorithmic(self):
+        """Per-launch algorithmic work of each stage (flops for the GEMM, bytes for the transforms)."""
+        T = self.plan.T
+        return {
+            "kt_bytes": 4.0 * self.K * self.C * (9 + 64),
+            "it_bytes": 4.0 * self.N * self.C * self.H * self.H + 256.0 * self.C * T,
+            "gemm_flops": 2.0 * 64 * self.K * self.C * T,
+            "ot_bytes": 256.0 * self.K * T + 4.0 * self.N * self.K * self.H * self.H,
+        }
+
+
+def forward(L, lay, V, M):
+    L.wino_forward(lay.plan, lay.x, lay.w, lay.U, V, M, lay.y)
+
+
+def tune_layer(L, lay, V, M, scratch_bytes, iters=3):
+    """Pick the GEMM tile shape with the shortest whole-layer forward."""
+    best = (None, 1e30)
+    for cfg in L.wino_configs():
+        plan = L.wino_plan(lay.shape, cfg.id)
+        if plan.V_bytes > scratch_bytes[0] or plan.M_bytes > scratch_bytes[1]:
+            continue
+        if plan.K_pad > 2 * lay.K and cfg.bm > 32:
+            continue
+        lay.plan = plan
+        mark = L.mark()
+        lay.U = L.alloc(plan.U_bytes)
+        forward(L, lay, V, M)
+        L.sync()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            forward(L, lay, V, M)
+        L.sync()
+        ms = (time.perf_counter() - t0) / iters * 1e3
+        L.release(mark)
+        if ms < best[1]:
+            best = (cfg.id, ms)
+    return best
+
+
+def cpu_baseline(target_seconds=12.0):
+    """Naive direct convolution (the oracle's restatement of the reference's
+    ConvNaiveLayer, OpenMP over images x output channels) on the VGG-16 stack."""
+    from oracle import oracle as O
+    cores = O.lib().fco_num_threads()
+
+    def run(batch):
+        total_flops, total_s = 0.0, 0.0
+        for (C, K, H, rep) in VGG16:
+            s = O.shape(batch, C, H, H, K)
+            x, w = O.make_inputs(s, seed=0)
+            t0 = time.perf_counter()
+            O.naive_conv_f32(s, x, w)
+            dt = time.perf_counter() - t0
+            total_flops += 2.0 * batch * K * C * H * H * 9 * rep
+            total_s += dt * rep
+        return total_flops, total_s
+
+    fl, s1 = run(1)
+    batch = int(max(1, min(32, target_seconds // max(s1, 1e-3))))
+    if batch > 1:
+        fl, s1 = run(batch)
+    return {"value": round(fl / s1 / 1e9, 2), "unit": "GFLOP/s", "cores": cores, "kind": "port",
+            "sample": "naive direct conv (restatement of the reference's ConvNaiveLayer; the reference's NEON "
+                      "kernels do not build on this x86 host), VGG-16 13-layer conv stack at batch %d, %.1f s"
+                      % (batch, s1)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="vgg16_b32", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-tune", action="store_true", help="use the built-in default tile shape per layer")
+    ap.add_argument("--offline-filter", action="store_true",
+                    help="transform the filters once outside the timed region")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--stage-events", default="all", choices=["all", "gemm", "none"],
+                    help="which kernels are bracketed by events inside the timed region")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (the layers shard by batch with no exchange step; "
+              "see DESIGN.md); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import fastconv_amd as F
+    layers_def, N, desc = WORKLOADS[args.workload]
+    rng = np.random.default_rng(0)
+
+    # arena: activations + filters + U per layer, one shared V and M (largest layer)
+    act = sum(4 * N * (C + K) * H * H for (C, K, H, _) in layers_def)
+    tiles = lambda H: N * ((H + 5) // 6) ** 2
+    vmax = max(256 * (C + 32) * (tiles(H) + 256) for (C, K, H, _) in layers_def)
+    mmax = max(256 * max(2 * K if K < 128 else K + 128, 128) * (tiles(H) + 256) for (C, K, H, _) in layers_def)
+    umax = sum(256 * (C + 32) * (K + 256) for (C, K, H, _) in layers_def) * 2
+    pool = int(act + vmax + mmax + umax + (512 << 20))
+    L = F.load(0, pool)
+    info = L.device_info()
+    log("device:", info)
+    V, M = L.alloc(vmax), L.alloc(mmax)
+    layers = [Layer(L, F, N, C, K, H, rep, rng) for (C, K, H, rep) in layers_def]
+
+    # tile shape per layer
+    for lay in layers:
+        if args.no_tune:
+            cfg, ms = 0, 0.0
+            for c in L.wino_configs():     # first configuration that does not over-pad K
+                if L.wino_plan(lay.shape, c.id).K_pad < 2 * lay.K or c.bm == 32:
+                    cfg = c.id
+                    break
+        else:
+            cfg, ms = tune_layer(L, lay, V, M, (vmax, mmax))
+        lay.plan = L.wino_plan(lay.shape, cfg)
+        lay.U = L.alloc(lay.plan.U_bytes)
+        L.wino_filter_transform(lay.plan, lay.w, lay.U)
+        g = L.wino_configs()[cfg]
+        log("layer %d->%d @%d: tile %dx%dx%d (cfg %d) %.3f ms" % (lay.C, lay.K, lay.H, g.bm, g.bn, g.bk, cfg, ms))
+    L.sync()
+
+    filter_ready = args.offline_filter
+
+    def step():
+        for lay in layers:
+            for _ in range(lay.repeats):
+                L.wino_forward(lay.plan, lay.x, lay.w, lay.U, V, M, lay.y, filter_ready=filter_ready)
+
+    for _ in range(args.warmup):
+        step()
+    L.sync()
+
+    mask = {"all": 0x0f, "gemm": 1 << ST_GEMM, "none": 0}[args.stage_events]
+    L.timing(mask)
+    L.timing_reset()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    L.sync()
+    elapsed = time.perf_counter() - t0
+    stage = [L.stage_time(i) for i in range(4)]
+    L.timing(0)
+
+    ms_per_step = elapsed / args.steps * 1e3
+    step_flops = sum(l.flops * l.repeats for l in layers)
+    value = step_flops / (ms_per_step * 1e-3) / 1e9
+
+    # dominant kernel: the batched GEMM. achieved = algorithmic flops of all its launches / their event time
+    gemm_flops_step = sum(l.algorithmic()["gemm_flops"] * l.repeats for l in layers)
+    launches_step = sum(l.repeats for l in layers)
+    roofline = {"kernel": "wino_gemm_kernel", "bound": "mfma", "achieved": None, "peak": PEAK_MFMA_F32_TFLOPS,
+                "unit": "TFLOP/s", "frac": None, "traffic": None}
+    if stage[ST_GEMM][1] > 0:
+        gemm_ms, gemm_cnt = stage[ST_GEMM]
+        ach = gemm_flops_step * (gemm_cnt / launches_step) / (gemm_ms * 1e-3) / 1e12
+        roofline.update(achieved=round(ach, 2), frac=round(ach / PEAK_MFMA_F32_TFLOPS, 4),
+                        launches=gemm_cnt, avg_launch_ms=round(gemm_ms / gemm_cnt, 5),
+                        flops_per_launch_avg=gemm_flops_step / launches_step)
+    transforms = {}
+    for name, idx, key in (("input_transform", ST_IT, "it_bytes"), ("output_transform", ST_OT, "ot_bytes"),
+                           ("filter_transform", ST_KT, "kt_bytes")):
+        ms, cnt = stage[idx]
+        if cnt > 0:
+            b = sum(l.algorithmic()[key] * l.repeats for l in layers) * (cnt / launches_step)
+            gbs = b / (ms * 1e-3) / 1e9
+            transforms[name] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                "frac": round(gbs / PEAK_HBM_GBS, 4), "launches": cnt}
+
+    # per-layer detail, outside the timed region
+    per_layer = []
+    L.timing(0x0f)
+    for lay in layers:
+        L.timing_reset()
+        reps = 5
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            forward(L, lay, V, M)
+        L.sync()
+        st = [L.stage_time(i)[0] / reps for i in range(4)]
+        total = sum(st)
+        a = lay.algorithmic()
+        g = L.wino_configs()[lay.plan.gemm_config]
+        per_layer.append({
+            "layer": "%d->%d@%d" % (lay.C, lay.K, lay.H), "batch": N, "repeats": lay.repeats,
+            "tile": "%dx%dx%d" % (g.bm, g.bn, g.bk), "ms": round(total, 4),
+            "gflops": round(lay.flops / (total * 1e-3) / 1e9, 1),
+            "gemm_tflops": round(a["gemm_flops"] / (st[ST_GEMM] * 1e-3) / 1e12, 2),
+            "gemm_frac_mfma": round(a["gemm_flops"] / (st[ST_GEMM] * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 3),
+            "input_tran_gbs": round(a["it_bytes"] / (st[ST_IT] * 1e-3) / 1e9, 0),
+            "output_tran_gbs": round(a["ot_bytes"] / (st[ST_OT] * 1e-3) / 1e9, 0),
+            "stage_ms": {"kernel_tran": round(st[ST_KT], 4), "input_tran": round(st[ST_IT], 4),
+                         "gemm": round(st[ST_GEMM], 4), "output_tran": round(st[ST_OT], 4)},
+        })
+    L.timing(0)
+
+    out = {
+        "metric": "effective GFLOP/s over the conv stack (direct-conv FLOP count / time)",
+        "value": round(value, 1), "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": args.workload, "description": desc, "batch": N, "algorithm": "winograd_f63_staged",
+                   "filter_transform": "offline" if filter_ready else "online (inside the timed region)",
+                   "tuned": not args.no_tune, "stage_events": args.stage_events,
+                   "device": info["arch"], "compute_units": info["compute_units"], "clock_mhz": info["clock_mhz"]},
+        "roofline": roofline,
+        "transform_rooflines": transforms,
+        "layers": per_layer,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    L.close()
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

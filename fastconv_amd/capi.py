@@ -154,6 +154,14 @@ class Library:
         self._check(self.c.fc_pool_alloc(self.pool, nbytes, C.byref(p)))
         return p
 
+    def mark(self):
+        m = C.c_size_t()
+        self._check(self.c.fc_pool_mark(self.pool, C.byref(m)))
+        return m.value
+
+    def release(self, mark):
+        self._check(self.c.fc_pool_release(self.pool, mark))
+
     def reset_pool(self):
         self._check(self.c.fc_pool_reset(self.pool))
 
@@ -189,7 +197,9 @@ class Library:
 
     # ---- timing
     def timing(self, on):
-        self._check(self.c.fc_timing_enable(self.ctx, 1 if on else 0))
+        """on: False/0 off, True all stages, or a bit mask of (1 << stage)."""
+        mask = 0x7f if on is True else int(on)
+        self._check(self.c.fc_timing_enable(self.ctx, mask))
 
     def timing_reset(self):
         self._check(self.c.fc_timing_reset(self.ctx))

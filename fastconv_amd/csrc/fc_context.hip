@@ -48,7 +48,7 @@ extern "C" int fc_init(int device, fc_context **out) {
     if (!ctx) return FC_ERR_OOM;
     ctx->magic = FC_CTX_MAGIC;
     ctx->device = device;
-    ctx->timing = false;
+    ctx->timing_mask = 0;
     ctx->stream = nullptr;
     memset(ctx->stage_ms, 0, sizeof ctx->stage_ms);
     memset(ctx->stage_launches, 0, sizeof ctx->stage_launches);
@@ -254,7 +254,7 @@ static hipEvent_t fc_take_event(fc_context *ctx) {
 }
 
 fc_stage_scope::fc_stage_scope(fc_context *c, int stage) : ctx(c), stop(nullptr), active(false) {
-    if (!c->timing) return;
+    if (!(c->timing_mask & (1u << stage))) return;
     if (c->pending.size() >= 8192) (void)fc_timing_fold(c);
     hipEvent_t start = fc_take_event(c);
     stop = fc_take_event(c);
@@ -268,13 +268,13 @@ fc_stage_scope::~fc_stage_scope() {
     if (active) (void)hipEventRecord(stop, ctx->stream);
 }
 
-extern "C" int fc_timing_enable(fc_context *ctx, int on) {
+extern "C" int fc_timing_enable(fc_context *ctx, int stage_mask) {
     if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
-    if (!on) {
+    if (!stage_mask) {
         const int rc = fc_timing_fold(ctx);
         if (rc) return rc;
     }
-    ctx->timing = on != 0;
+    ctx->timing_mask = (unsigned)stage_mask & ((1u << FC_STAGE_COUNT) - 1);
     return FC_OK;
 }
 

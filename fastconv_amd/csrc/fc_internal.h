@@ -19,7 +19,7 @@ struct fc_context {
     hipStream_t stream;
     hipDeviceProp_t props;
     std::string last_error;
-    bool timing;
+    unsigned timing_mask;   // bit s set: launches of stage s are bracketed by events
     std::vector<hipEvent_t> free_events;
     std::vector<fc_timing_pair> pending;
     double stage_ms[FC_STAGE_COUNT];

@@ -111,7 +111,7 @@ int ConvIm2colLayer::Forward() {
     d.Check(fc_sync(d.ctx()), "fc_sync");
     total.accumBench();
 
-    d.Check(fc_timing_enable(d.ctx(), 1), "fc_timing_enable");
+    d.Check(fc_timing_enable(d.ctx(), FC_TIMING_ALL), "fc_timing_enable");
     d.Check(fc_timing_reset(d.ctx()), "fc_timing_reset");
     for (size_t i = 0; i < iterations; i++) RunOnce();
     double ms = 0;

@@ -185,7 +185,7 @@ int ConvWinoF63Layer::Forward() {
     d.Check(fc_sync(d.ctx()), "fc_sync");
     total.accumBench();
 
-    d.Check(fc_timing_enable(d.ctx(), 1), "fc_timing_enable");
+    d.Check(fc_timing_enable(d.ctx(), FC_TIMING_ALL), "fc_timing_enable");
     d.Check(fc_timing_reset(d.ctx()), "fc_timing_reset");
     for (size_t i = 0; i < iterations; i++) RunOnce();
     const int stages[4] = {FC_STAGE_INPUT_TRAN, FC_STAGE_KERNEL_TRAN, FC_STAGE_TENSOR_GEMM, FC_STAGE_OUTPUT_TRAN};

@@ -101,11 +101,13 @@ int fc_fill_zero(fc_context *ctx, void *dst_dev, size_t bytes);
 
 /* ---- stage timing (utility/helper.h:66-80 Timer, per stage) ----------- */
 
-/* When enabled, every kernel launch below is bracketed by two events on the
- * context's stream.  fc_stage_time_ms() waits for the stream, folds the pending
- * event pairs into per-stage totals and returns total milliseconds and launch
- * count since the last fc_timing_reset(). */
-int fc_timing_enable(fc_context *ctx, int on);
+/* stage_mask has bit (1 << stage) set for every stage whose kernel launches are
+ * to be bracketed by two events on the context's stream (FC_TIMING_ALL for all,
+ * 0 to switch timing off).  fc_stage_time_ms() waits for the stream, folds the
+ * pending event pairs into per-stage totals and returns total milliseconds and
+ * launch count since the last fc_timing_reset(). */
+#define FC_TIMING_ALL 0x7f
+int fc_timing_enable(fc_context *ctx, int stage_mask);
 int fc_timing_reset(fc_context *ctx);
 int fc_stage_time_ms(fc_context *ctx, int stage, double *total_ms, long *launches);
 
