@@ -10,6 +10,7 @@
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));   // native vector: arrays of it stay in registers
 
 // Row table entry for reduction index kred = (c*kh + r)*kw + s:
 //   [2*kred]   = c*H*W + r*W + s      (offset from the window origin)
@@ -91,7 +92,7 @@ __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmPara
         xwin = p.x + (size_t)n * p.C * p.H * p.W + (long)ih0 * p.W + iw0;
     }
 
-    float4 ra[TL::A_LD];
+    floatx4 ra[TL::A_LD];
     float rb[TL::B_LD];
 
     auto load_global = [&](int k0) {
@@ -100,7 +101,7 @@ __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmPara
             const int v = tid + i * TL::THREADS;
             if (TL::A_VEC % TL::THREADS == 0 || v < TL::A_VEC) {
                 const int row = v / (BM / 4), col = (v % (BM / 4)) * 4;
-                ra[i] = *reinterpret_cast<const float4 *>(Ag + (size_t)(k0 + row) * p.K_pad + col);
+                ra[i] = *reinterpret_cast<const floatx4 *>(Ag + (size_t)(k0 + row) * p.K_pad + col);
             }
         }
 #pragma unroll
@@ -118,7 +119,7 @@ __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmPara
             const int v = tid + i * TL::THREADS;
             if (TL::A_VEC % TL::THREADS == 0 || v < TL::A_VEC) {
                 const int row = v / (BM / 4), col = (v % (BM / 4)) * 4;
-                *reinterpret_cast<float4 *>(&As[buf][row][col]) = ra[i];
+                *reinterpret_cast<floatx4 *>(&As[buf][row][col]) = ra[i];
             }
         }
 #pragma unroll

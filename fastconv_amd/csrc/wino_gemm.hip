@@ -4,11 +4,28 @@
 // fastest, which is exactly the order v_mfma_f32_32x32x2_f32 wants its lanes in
 // (lane l holds row/col l%32 of reduction step l/32), so tiles go global -> LDS
 // as straight 16-byte copies and LDS -> registers as conflict-free dword reads.
+#include <utility>
+
 #include "fc_internal.h"
 
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// Copy passes written as pack expansions, so that every register-array index is a
+// literal constant: with a loop index the arrays are not promoted to registers
+// and the tile makes a round trip through scratch memory.
+template <int... I>
+__device__ __forceinline__ void load_rows(floatx4 (&r)[sizeof...(I)], const float *p, size_t rowStride,
+                                          std::integer_sequence<int, I...>) {
+    ((r[I] = *reinterpret_cast<const floatx4 *>(p + (size_t)I * rowStride)), ...);
+}
+template <int... I>
+__device__ __forceinline__ void store_rows(float *lds, const floatx4 (&r)[sizeof...(I)], int rowStride,
+                                           std::integer_sequence<int, I...>) {
+    ((*reinterpret_cast<floatx4 *>(lds + I * rowStride) = r[I]), ...);
+}
 
 // Workgroup tile BM x BN x BK; WGM x WGN wavefronts, each owning
 // (BM/WGM) x (BN/WGN) of the tile as 32x32 MFMA blocks.
@@ -18,12 +35,13 @@ struct GemmTile {
     static constexpr int WM = BM / WGM, WN = BN / WGN;
     static constexpr int MI = WM / 32, NI = WN / 32;
     static constexpr int A_VEC = BK * BM / 4, B_VEC = BK * BN / 4;      // float4 per stage
-    static constexpr int A_LD = (A_VEC + THREADS - 1) / THREADS;
-    static constexpr int B_LD = (B_VEC + THREADS - 1) / THREADS;
+    static constexpr int A_LD = A_VEC / THREADS, B_LD = B_VEC / THREADS;
+    static constexpr int A_ROWS = THREADS * 4 / BM, B_ROWS = THREADS * 4 / BN;   // tile rows per copy pass
     static constexpr int LDS_BYTES = 2 * BK * (BM + BN) * 4;
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be whole 32x32 MFMA blocks");
     static_assert(BK % 2 == 0, "32x32x2 MFMA consumes two reduction steps");
-    static_assert(BM % 4 == 0 && BN % 4 == 0, "16-byte copies");
+    static_assert(A_VEC % THREADS == 0 && B_VEC % THREADS == 0, "every thread copies the same number of float4");
+    static_assert(A_LD >= 1 && B_LD >= 1, "tile smaller than one copy pass");
 };
 
 // Workgroups are dealt to the 8 XCDs round-robin by linear id.  All tiles of one
@@ -37,8 +55,9 @@ __global__ __launch_bounds__(TL::THREADS) void wino_gemm_kernel(const float *__r
                                                                 float *__restrict__ M, int K_pad, int C_pad,
                                                                 int T_pad, int nKB, int nTB) {
     constexpr int BM = TL::BM_, BN = TL::BN_, BK = TL::BK_;
-    __shared__ __attribute__((aligned(16))) float As[2][BK][BM];
-    __shared__ __attribute__((aligned(16))) float Bs[2][BK][BN];
+    constexpr int MI = TL::MI, NI = TL::NI, A_LD = TL::A_LD, B_LD = TL::B_LD;
+    __shared__ __attribute__((aligned(16))) float As[2][BK * BM];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK * BN];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm0 = (wave / TL::WGN_) * TL::WM, wn0 = (wave % TL::WGN_) * TL::WN;
@@ -49,88 +68,88 @@ __global__ __launch_bounds__(TL::THREADS) void wino_gemm_kernel(const float *__r
     const int f = fl * 8 + xcd;
     const int tb = rem / nKB, kb = rem - tb * nKB;
 
-    const float *Ag = U + (size_t)f * C_pad * K_pad + (size_t)kb * BM;
-    const float *Bg = V + (size_t)f * C_pad * T_pad + (size_t)tb * BN;
+    // this thread's float4 of each copy pass: row r0 + i*ROWS, column c4
+    const int arow = tid / (BM / 4), acol = (tid % (BM / 4)) * 4;
+    const int brow = tid / (BN / 4), bcol = (tid % (BN / 4)) * 4;
+    const float *ag = U + ((size_t)f * C_pad + arow) * K_pad + (size_t)kb * BM + acol;
+    const float *bg = V + ((size_t)f * C_pad + brow) * T_pad + (size_t)tb * BN + bcol;
+    const size_t aStage = (size_t)BK * K_pad, bStage = (size_t)BK * T_pad;
+    const int aLds = arow * BM + acol, bLds = brow * BN + bcol;
 
-    float4 ra[TL::A_LD], rb[TL::B_LD];
+    using SeqA = std::make_integer_sequence<int, A_LD>;
+    using SeqB = std::make_integer_sequence<int, B_LD>;
+    const size_t aPass = (size_t)TL::A_ROWS * K_pad, bPass = (size_t)TL::B_ROWS * T_pad;
+    floatx4 ra[A_LD], rb[B_LD];
+    load_rows(ra, ag, aPass, SeqA());
+    load_rows(rb, bg, bPass, SeqB());
 
-    auto load_global = [&](int c0) {
+    floatx16 acc[MI][NI];
 #pragma unroll
-        for (int i = 0; i < TL::A_LD; i++) {
-            const int v = tid + i * TL::THREADS;
-            if (TL::A_VEC % TL::THREADS == 0 || v < TL::A_VEC) {
-                const int row = v / (BM / 4), col = (v % (BM / 4)) * 4;
-                ra[i] = *reinterpret_cast<const float4 *>(Ag + (size_t)(c0 + row) * K_pad + col);
-            }
-        }
+    for (int mi = 0; mi < MI; mi++)
 #pragma unroll
-        for (int i = 0; i < TL::B_LD; i++) {
-            const int v = tid + i * TL::THREADS;
-            if (TL::B_VEC % TL::THREADS == 0 || v < TL::B_VEC) {
-                const int row = v / (BN / 4), col = (v % (BN / 4)) * 4;
-                rb[i] = *reinterpret_cast<const float4 *>(Bg + (size_t)(c0 + row) * T_pad + col);
-            }
-        }
-    };
-    auto store_lds = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < TL::A_LD; i++) {
-            const int v = tid + i * TL::THREADS;
-            if (TL::A_VEC % TL::THREADS == 0 || v < TL::A_VEC) {
-                const int row = v / (BM / 4), col = (v % (BM / 4)) * 4;
-                *reinterpret_cast<float4 *>(&As[buf][row][col]) = ra[i];
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < TL::B_LD; i++) {
-            const int v = tid + i * TL::THREADS;
-            if (TL::B_VEC % TL::THREADS == 0 || v < TL::B_VEC) {
-                const int row = v / (BN / 4), col = (v % (BN / 4)) * 4;
-                *reinterpret_cast<float4 *>(&Bs[buf][row][col]) = rb[i];
-            }
-        }
-    };
-
-    floatx16 acc[TL::MI][TL::NI];
-#pragma unroll
-    for (int mi = 0; mi < TL::MI; mi++)
-#pragma unroll
-        for (int ni = 0; ni < TL::NI; ni++)
+        for (int ni = 0; ni < NI; ni++)
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[mi][ni][i] = 0.f;
 
-    load_global(0);
-    store_lds(0);
+    store_rows(&As[0][aLds], ra, TL::A_ROWS * BM, SeqA());
+    store_rows(&Bs[0][bLds], rb, TL::B_ROWS * BN, SeqB());
     __syncthreads();
 
+    // fragment addresses: lane l reads element (row kk + l/32, column base + l%32)
     const int lrow = lane >> 5, lcol = lane & 31;
+    const int aFrag = lrow * BM + wm0 + lcol, bFrag = lrow * BN + wn0 + lcol;
     const int nStages = C_pad / BK;
     for (int s = 0; s < nStages; s++) {
-        const int cur = s & 1;
-        if (s + 1 < nStages) load_global((s + 1) * BK);
+        const float *as = As[s & 1], *bs = Bs[s & 1];
+        const bool more = s + 1 < nStages;
+        if (more) {
+            ag += aStage;
+            bg += bStage;
+            load_rows(ra, ag, aPass, SeqA());
+            load_rows(rb, bg, bPass, SeqB());
+        }
+        // the fragments of step kk+2 are fetched from LDS before the MFMAs of step kk are issued
+        float a[2][MI], bb[2][NI];
+#pragma unroll
+        for (int mi = 0; mi < MI; mi++) a[0][mi] = as[aFrag + mi * 32];
+#pragma unroll
+        for (int ni = 0; ni < NI; ni++) bb[0][ni] = bs[bFrag + ni * 32];
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 2) {
-            float a[TL::MI], bb[TL::NI];
+            const int cur = (kk >> 1) & 1, nxt = cur ^ 1;
+            if (kk + 2 < BK) {
 #pragma unroll
-            for (int mi = 0; mi < TL::MI; mi++) a[mi] = As[cur][kk + lrow][wm0 + mi * 32 + lcol];
+                for (int mi = 0; mi < MI; mi++) a[nxt][mi] = as[aFrag + (kk + 2) * BM + mi * 32];
 #pragma unroll
-            for (int ni = 0; ni < TL::NI; ni++) bb[ni] = Bs[cur][kk + lrow][wn0 + ni * 32 + lcol];
+                for (int ni = 0; ni < NI; ni++) bb[nxt][ni] = bs[bFrag + (kk + 2) * BN + ni * 32];
+            }
 #pragma unroll
-            for (int mi = 0; mi < TL::MI; mi++)
+            for (int mi = 0; mi < MI; mi++)
 #pragma unroll
-                for (int ni = 0; ni < TL::NI; ni++)
-                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[mi], bb[ni], acc[mi][ni], 0, 0, 0);
+                for (int ni = 0; ni < NI; ni++)
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][mi], bb[cur][ni], acc[mi][ni], 0, 0, 0);
         }
-        if (s + 1 < nStages) store_lds(cur ^ 1);
+        // scheduling: after the first MFMA of a step, issue the LDS reads of the next step,
+        // so that their latency is covered by the remaining MFMAs
+#pragma unroll
+        for (int kk = 0; kk + 2 < BK; kk += 2) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, MI + NI, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, MI * NI - 1, 0);
+        }
+        if (more) {
+            store_rows(&As[(s & 1) ^ 1][aLds], ra, TL::A_ROWS * BM, SeqA());
+            store_rows(&Bs[(s & 1) ^ 1][bLds], rb, TL::B_ROWS * BN, SeqB());
+        }
         __syncthreads();
     }
 
     // D block layout: register i of lane l is row 8*(i/4) + 4*(l/32) + i%4, column l%32.
     float *Mg = M + ((size_t)f * K_pad + (size_t)kb * BM + wm0) * T_pad + (size_t)tb * BN + wn0;
 #pragma unroll
-    for (int mi = 0; mi < TL::MI; mi++)
+    for (int mi = 0; mi < MI; mi++)
 #pragma unroll
-        for (int ni = 0; ni < TL::NI; ni++)
+        for (int ni = 0; ni < NI; ni++)
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 const int row = mi * 32 + 8 * (i / 4) + 4 * lrow + (i % 4);
