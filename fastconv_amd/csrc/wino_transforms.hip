@@ -97,97 +97,112 @@ __global__ __launch_bounds__(256) void wino_filter_transform_kernel(const float 
 
 // ----------------------------------------------------------------- input
 
+// Tiles are numbered t = (n*tH + th)*tW + tw, so t / tW is a "band": one row of
+// tiles of one image, gb = n*tH + th.  Both transform kernels give a workgroup
+// TPB consecutive tiles starting at a multiple of TPB, whatever bands and images
+// that range crosses: every store to (or load from) a frequency plane is then a
+// whole number of aligned 128-byte lines.
 struct InTParams {
     const float *x;
     float *V;
     int N, C, H, W, pad_t, pad_l;
-    int tH, tW, tileN;
-    long T;
+    int tH, tW;
+    long T;          // real tiles; tiles in [T, T_pad) are written as zeros
     int C_pad;
     long T_pad;
-    int P, R;        // images and tile rows ("bands") per block; a block always spans all tW columns
-    int nPG, nBG;    // groups of images, groups of bands
-    int LW;          // 6*tW + 2 columns of the band as the tiles see it (incl. padding columns)
-    fc_fastdiv divLW, divR, divTW;
+    int LW;          // 6*tW + 2: columns of a band as its tiles see it, padding columns included
+    fc_fastdiv divLW, divTH, divTW;
 };
 
-// Block = one input channel x (P images x R bands x tW tiles), TPB tiles at most.
-// Pass 1 applies B^T down the 8 rows of each band: a thread owns one column of
-// one band, so the 8 global loads of a wavefront are row-contiguous.  Pass 2
-// applies B along the rows from LDS: a thread owns one tile (and 8*TPB/256 of
-// its 8 rows) and stores to the frequency planes with lanes on consecutive
-// tiles.  The extra last block in x zero-fills the tile padding [T, T_pad).
-template <int TPB>
+// Block = one input channel x TPB consecutive tiles.
+// Pass 1 applies B^T down the 8 rows of each band the tile range touches: a
+// thread owns up to ITEMS columns (one column of one band each), so the 8 global loads of a wavefront are
+// row-contiguous.  Pass 2 applies B along the rows out of LDS: a thread owns one
+// tile and 8*TPB/256 of its 8 rows, and stores to the frequency planes with lanes
+// on consecutive tiles.
+template <int TPB, int ITEMS>
 __global__ __launch_bounds__(256) void wino_input_transform_kernel(const InTParams p) {
-    extern __shared__ float lds[];   // [P*R][8][LW]
+    extern __shared__ float lds[];   // [bands][8][LW]
     const int tid = threadIdx.x;
     const int c = blockIdx.y;
     const size_t plane = (size_t)p.C_pad * p.T_pad;
-    const int nChunks = p.nPG * p.nBG;
-
-    if ((int)blockIdx.x == nChunks) {
-        const long padT = p.T_pad - p.T;
-        for (long e = tid; e < padT * 64; e += 256) {
-            const long f = e / padT, t = p.T + (e - f * padT);
-            p.V[f * plane + (size_t)c * p.T_pad + t] = 0.f;
-        }
-        return;
-    }
-    const int pg = blockIdx.x / p.nBG, bg = blockIdx.x - pg * p.nBG;
-    const int n0 = pg * p.P, th0 = bg * p.R;
-    const int PR = p.P * p.R;
+    const uint32_t t0 = blockIdx.x * TPB;
+    const uint32_t tLast = min((uint32_t)(t0 + TPB), (uint32_t)p.T) - 1;   // last real tile (wraps if none)
+    const bool anyReal = t0 < (uint32_t)p.T;
+    const uint32_t gb0 = fc_div(t0, p.divTW), gbL = anyReal ? fc_div(tLast, p.divTW) : gb0;
+    const int tw0 = t0 - gb0 * p.tW, twL = tLast - gbL * p.tW;
+    const int NB = anyReal ? (int)(gbL - gb0) + 1 : 0;
 
     if (c < p.C) {
-        const int items = PR * p.LW;
-        for (int e = tid; e < items; e += 256) {
-            const int pr = fc_div(e, p.divLW), lx = e - pr * p.LW;
-            const int pp = fc_div(pr, p.divR), r = pr - pp * p.R;
-            const int n = n0 + pp, th = th0 + r;
-            if (n >= p.N || th >= p.tH) continue;
-            const int gx = lx - p.pad_l, gy0 = th * 6 - p.pad_t;
-            float d[8], o[8];
-            const bool colOK = gx >= 0 && gx < p.W;
-            const float *src = p.x + (((size_t)n * p.C + c) * p.H) * p.W + gx;
+        // All global loads of a thread (up to ITEMS columns x 8 rows) are issued before any
+        // is consumed: the kernel is latency-bound otherwise (few bytes in flight per CU).
+        const int items = NB * p.LW;
+        float d[ITEMS][8];
+        int dstOff[ITEMS];
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const int gy = gy0 + i;
-                d[i] = (colOK && gy >= 0 && gy < p.H) ? src[(long)gy * p.W] : 0.f;
+        for (int it = 0; it < ITEMS; it++) {
+            const int e = tid + it * 256;
+            dstOff[it] = -1;
+#pragma unroll
+            for (int i = 0; i < 8; i++) d[it][i] = 0.f;
+            if (e < items) {
+                const int j = fc_div(e, p.divLW), lx = e - j * p.LW;
+                // columns this block needs of band j
+                const int lxA = (j == 0) ? tw0 * 6 : 0, lxB = (j == NB - 1) ? twL * 6 + 8 : p.LW;
+                if (lx >= lxA && lx < lxB) {
+                    dstOff[it] = j * 8 * p.LW + lx;
+                    const uint32_t gb = gb0 + j;
+                    const uint32_t n = fc_div(gb, p.divTH), th = gb - n * p.tH;
+                    const int gx = lx - p.pad_l, gy0 = (int)th * 6 - p.pad_t;
+                    if (gx >= 0 && gx < p.W) {
+                        const float *src = p.x + (((size_t)n * p.C + c) * p.H) * p.W + gx;
+#pragma unroll
+                        for (int i = 0; i < 8; i++) {
+                            const int gy = gy0 + i;
+                            if (gy >= 0 && gy < p.H) d[it][i] = src[(long)gy * p.W];
+                        }
+                    }
+                }
             }
-            bt8(d, o);
-            float *dstl = lds + (size_t)pr * 8 * p.LW + lx;
+        }
 #pragma unroll
-            for (int i = 0; i < 8; i++) dstl[i * p.LW] = o[i];
+        for (int it = 0; it < ITEMS; it++) {
+            if (dstOff[it] >= 0) {
+                float o[8];
+                bt8(d[it], o);
+                float *dstl = lds + dstOff[it];
+#pragma unroll
+                for (int i = 0; i < 8; i++) dstl[i * p.LW] = o[i];
+            }
         }
     }
     __syncthreads();
 
     constexpr int IPT = 8 * TPB / 256;     // rows of the 8x8 tile per thread
     const int tl = tid % TPB, ig = tid / TPB;
-    const int pr = fc_div(tl, p.divTW), q = tl - pr * p.tW;
-    if (pr >= PR) return;
-    const int pp = fc_div(pr, p.divR), r = pr - pp * p.R;
-    const int n = n0 + pp, th = th0 + r;
-    if (n >= p.N || th >= p.tH) return;
-    const long t = (long)n * p.tileN + (long)th * p.tW + q;
+    const uint32_t t = t0 + tl;
     float *dst = p.V + (size_t)c * p.T_pad + t;
-    if (c < p.C) {
+    if (c < p.C && t < (uint32_t)p.T) {
+        const uint32_t gb = fc_div(t, p.divTW);
+        const int q = t - gb * p.tW, j = gb - gb0;
 #pragma unroll
         for (int ii = 0; ii < IPT; ii++) {
             const int i = ig * IPT + ii;
-            const float *row = lds + ((size_t)pr * 8 + i) * p.LW + q * 6;
+            const float *row = lds + ((size_t)j * 8 + i) * p.LW + q * 6;
             float d[8], o[8];
 #pragma unroll
-            for (int j = 0; j < 8; j++) d[j] = row[j];
+            for (int jj = 0; jj < 8; jj++) d[jj] = row[jj];
             bt8(d, o);
 #pragma unroll
-            for (int j = 0; j < 8; j++) dst[(size_t)(i * 8 + j) * plane] = o[j];
+            for (int jj = 0; jj < 8; jj++) dst[(size_t)(i * 8 + jj) * plane] = o[jj];
         }
     } else {
+        // padding channel or padding tile: the GEMM reads it, so it must be zero
 #pragma unroll
         for (int ii = 0; ii < IPT; ii++) {
             const int i = ig * IPT + ii;
 #pragma unroll
-            for (int j = 0; j < 8; j++) dst[(size_t)(i * 8 + j) * plane] = 0.f;
+            for (int jj = 0; jj < 8; jj++) dst[(size_t)(i * 8 + jj) * plane] = 0.f;
         }
     }
 }
@@ -199,90 +214,94 @@ struct OutTParams {
     const float *bias;
     float *y;
     int N, K, OH, OW, relu;
-    int tH, tW, tileN;
+    int tH, tW;
+    long T;
     int K_pad;
     long T_pad;
-    int P, R, nPG, nBG;
-    fc_fastdiv divR, divTW;
+    fc_fastdiv divTH, divTW;
 };
 
-// Block = one output channel x (P images x R bands x tW tiles); one thread per
-// tile.  The 64 plane loads of a wavefront are each 256 contiguous bytes.  The
-// 6x6 results are laid into LDS as the exact image rows they cover and copied
-// out as one contiguous run per image.
+// Block = one output channel x TPB consecutive tiles, one thread per tile.  The 64
+// plane loads of a wavefront are each 256 contiguous bytes.  The 6x6 results are
+// laid into LDS as the image rows they cover ([band][6][OW]) and copied out band
+// by band: a band the block covers completely is one contiguous run of rows*OW
+// floats, a partly covered band (first or last of the range) is one run per row.
 template <int TPB>
 __global__ __launch_bounds__(TPB) void wino_output_transform_kernel(const OutTParams p) {
-    extern __shared__ float lds[];   // [P][rows*OW]
-    const int tid = threadIdx.x;
+    extern __shared__ __attribute__((aligned(16))) float lds[];   // [bands][6][OW]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int k = blockIdx.y;
-    const int pg = blockIdx.x / p.nBG, bg = blockIdx.x - pg * p.nBG;
-    const int n0 = pg * p.P, th0 = bg * p.R;
-    const int row0 = th0 * 6;
-    const int rows = min(p.R * 6, p.OH - row0);      // output rows this block covers
-    const int L = rows * p.OW;                       // floats per image in this block
+    const uint32_t t0 = blockIdx.x * TPB;
+    if (t0 >= (uint32_t)p.T) return;
+    const uint32_t tLast = min((uint32_t)(t0 + TPB), (uint32_t)p.T) - 1;
+    const uint32_t gb0 = fc_div(t0, p.divTW), gbL = fc_div(tLast, p.divTW);
+    const int tw0 = t0 - gb0 * p.tW, twL = tLast - gbL * p.tW;
+    const int NB = (int)(gbL - gb0) + 1;
+    const int bandElems = 6 * p.OW;
 
-    const int pr = fc_div(tid, p.divTW), q = tid - pr * p.tW;
-    const int pp = fc_div(pr, p.divR), r = pr - pp * p.R;
-    const int n = n0 + pp, th = th0 + r;
-    if (pr < p.P * p.R && n < p.N && th < p.tH) {
+    const uint32_t t = t0 + tid;
+    if (t <= tLast) {
+        const uint32_t gb = fc_div(t, p.divTW);
+        const int q = t - gb * p.tW, j = gb - gb0;
         const size_t plane = (size_t)p.K_pad * p.T_pad;
-        const long t = (long)n * p.tileN + (long)th * p.tW + q;
         const float *src = p.M + (size_t)k * p.T_pad + t;
         float m[8][8];
 #pragma unroll
         for (int f = 0; f < 64; f++) m[f >> 3][f & 7] = src[(size_t)f * plane];
         float tmp[6][8];
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const float col[8] = {m[0][j], m[1][j], m[2][j], m[3][j], m[4][j], m[5][j], m[6][j], m[7][j]};
+        for (int jj = 0; jj < 8; jj++) {
+            const float col[8] = {m[0][jj], m[1][jj], m[2][jj], m[3][jj], m[4][jj], m[5][jj], m[6][jj], m[7][jj]};
             float s[6];
             at6(col, s);
 #pragma unroll
-            for (int i = 0; i < 6; i++) tmp[i][j] = s[i];
+            for (int i = 0; i < 6; i++) tmp[i][jj] = s[i];
         }
         const float b = p.bias ? p.bias[k] : 0.f;
-        float *img = lds + (size_t)pp * L;
-        const int colBase = q * 6;
+        float *img = lds + (size_t)j * bandElems + q * 6;
+        const int colsLeft = p.OW - q * 6;      // columns of this tile inside the image
 #pragma unroll
         for (int i = 0; i < 6; i++) {
             float s[6];
             at6(tmp[i], s);
-            const int lr = r * 6 + i;
-            if (lr < rows) {
 #pragma unroll
-                for (int j = 0; j < 6; j++) {
-                    float v = s[j] + b;
-                    if (p.relu) v = fmaxf(v, 0.f);
-                    if (colBase + j < p.OW) img[lr * p.OW + colBase + j] = v;
-                }
+            for (int jj = 0; jj < 6; jj++) {
+                float v = s[jj] + b;
+                if (p.relu) v = fmaxf(v, 0.f);
+                if (jj < colsLeft) img[i * p.OW + jj] = v;
             }
         }
     }
     __syncthreads();
-    const int nImg = min(p.P, p.N - n0);
-    const size_t imgStride = (size_t)p.K * p.OH * p.OW;
-    float *dst0 = p.y + ((size_t)n0 * p.K + k) * p.OH * p.OW + (size_t)row0 * p.OW;
-    for (int pi = 0; pi < nImg; pi++) {
-        const float *img = lds + (size_t)pi * L;
-        float *dst = dst0 + (size_t)pi * imgStride;
-        for (int e = tid; e < L; e += TPB) dst[e] = img[e];
+
+    constexpr int WAVES = TPB / 64;
+    const bool vec4 = (p.OW & 3) == 0;
+    for (int j = wave; j < NB; j += WAVES) {
+        const uint32_t gb = gb0 + j;
+        const uint32_t n = fc_div(gb, p.divTH), th = gb - n * p.tH;
+        const int rows = min(6, p.OH - (int)th * 6);
+        const int xA = (j == 0) ? tw0 * 6 : 0;
+        const int xB = min((j == NB - 1) ? (twL + 1) * 6 : p.tW * 6, p.OW);
+        float *dst = p.y + (((size_t)n * p.K + k) * p.OH + (size_t)th * 6) * p.OW;
+        const float *src = lds + (size_t)j * bandElems;
+        if (xA == 0 && xB == p.OW) {
+            const int len = rows * p.OW;
+            if (vec4) {
+                const float4 *s4 = reinterpret_cast<const float4 *>(src);
+                float4 *d4 = reinterpret_cast<float4 *>(dst);
+                for (int e = lane; e < len / 4; e += 64) d4[e] = s4[e];
+            } else {
+                for (int e = lane; e < len; e += 64) dst[e] = src[e];
+            }
+        } else {
+            for (int i = 0; i < rows; i++)
+                for (int x = xA + lane; x < xB; x += 64) dst[i * p.OW + x] = src[i * p.OW + x];
+        }
     }
 }
 
-// Choose images (P) and bands (R) per block for `tpb` tiles per block.
-bool chunking(int tpb, int N, int tH, int tW, int *P, int *R) {
-    const int tileN = tH * tW;
-    if (tW > tpb) return false;
-    if (tileN <= tpb) {
-        *R = tH;
-        *P = tpb / tileN;
-        if (*P > N) *P = N;
-    } else {
-        *P = 1;
-        *R = tpb / tW;
-    }
-    return true;
-}
+// Largest of 128 / 64 / 32 tiles per block that divides the padded tile count.
+int tiles_per_block(long T_pad) { return (T_pad % 128 == 0) ? 128 : (T_pad % 64 == 0) ? 64 : 32; }
 
 }  // namespace
 
@@ -345,37 +364,33 @@ extern "C" int fc_wino_input_transform(fc_context *ctx, const fc_wino_plan *plan
     InTParams p;
     p.x = x_dev; p.V = V_dev;
     p.N = s.N; p.C = s.C; p.H = s.H; p.W = s.W; p.pad_t = s.pt; p.pad_l = s.pl;
-    p.tH = plan->tiles_h; p.tW = plan->tiles_w; p.tileN = p.tH * p.tW;
+    p.tH = plan->tiles_h; p.tW = plan->tiles_w;
     p.T = plan->T; p.C_pad = plan->C_pad; p.T_pad = plan->T_pad;
     p.LW = 6 * p.tW + 2;
-    // pick the tiles-per-block variant that wastes the fewest lanes and fits 64 KiB of LDS
-    int best = 0, bestP = 0, bestR = 0;
-    double bestUtil = -1.0;
-    const int cand[3] = {64, 128, 256};
-    for (int i = 0; i < 3; i++) {
-        int P, R;
-        if (!chunking(cand[i], s.N, p.tH, p.tW, &P, &R)) continue;
-        const size_t ldsBytes = (size_t)P * R * 8 * p.LW * sizeof(float);
-        if (ldsBytes > 64 * 1024) continue;
-        const int nBG = (p.tH + R - 1) / R;
-        // average fraction of busy lanes over the band groups of one image group
-        const double util = (double)p.tH * p.tW * P / ((double)nBG * cand[i]);
-        if (util > bestUtil + 0.02) { bestUtil = util; best = cand[i]; bestP = P; bestR = R; }
-    }
-    if (!best) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_input_transform: image too wide", hipSuccess);
-    p.P = bestP; p.R = bestR;
-    p.nPG = (s.N + p.P - 1) / p.P;
-    p.nBG = (p.tH + p.R - 1) / p.R;
     p.divLW = fc_make_fastdiv(p.LW);
-    p.divR = fc_make_fastdiv(p.R);
+    p.divTH = fc_make_fastdiv(p.tH);
     p.divTW = fc_make_fastdiv(p.tW);
-    const size_t ldsBytes = (size_t)p.P * p.R * 8 * p.LW * sizeof(float);
-    const dim3 grid(p.nPG * p.nBG + 1, plan->C_pad);
+    const int tpb = tiles_per_block(plan->T_pad);
+    // a range of tpb tiles touches at most this many bands
+    const int maxBands = (tpb + p.tW - 2) / p.tW + 1;
+    const size_t ldsBytes = (size_t)maxBands * 8 * p.LW * sizeof(float);
+    if (ldsBytes > 64 * 1024) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_input_transform: image too wide", hipSuccess);
+    const dim3 grid((unsigned)(plan->T_pad / tpb), plan->C_pad);
     if (grid.y > 65535) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_input_transform: more than 65535 channels", hipSuccess);
     fc_stage_scope scope(ctx, FC_STAGE_INPUT_TRAN);
-    if (best == 64) wino_input_transform_kernel<64><<<grid, dim3(256), ldsBytes, ctx->stream>>>(p);
-    else if (best == 128) wino_input_transform_kernel<128><<<grid, dim3(256), ldsBytes, ctx->stream>>>(p);
-    else wino_input_transform_kernel<256><<<grid, dim3(256), ldsBytes, ctx->stream>>>(p);
+    // columns (band x column pairs) per thread in pass 1
+    const int itemsPerThread = (maxBands * p.LW + 255) / 256;
+    if (itemsPerThread > 6) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_input_transform: image too wide", hipSuccess);
+#define FC_LAUNCH_INT(TPB_)                                                                                    \
+    do {                                                                                                       \
+        if (itemsPerThread <= 2) wino_input_transform_kernel<TPB_, 2><<<grid, dim3(256), ldsBytes, ctx->stream>>>(p);      \
+        else if (itemsPerThread <= 4) wino_input_transform_kernel<TPB_, 4><<<grid, dim3(256), ldsBytes, ctx->stream>>>(p); \
+        else wino_input_transform_kernel<TPB_, 6><<<grid, dim3(256), ldsBytes, ctx->stream>>>(p);              \
+    } while (0)
+    if (tpb == 128) FC_LAUNCH_INT(128);
+    else if (tpb == 64) FC_LAUNCH_INT(64);
+    else FC_LAUNCH_INT(32);
+#undef FC_LAUNCH_INT
     FC_LAUNCH_CHECK(ctx, "wino_input_transform_kernel");
     return FC_OK;
 }
@@ -388,31 +403,20 @@ extern "C" int fc_wino_output_transform(fc_context *ctx, const fc_wino_plan *pla
     OutTParams p;
     p.M = M_dev; p.bias = bias_dev; p.y = y_dev;
     p.N = s.N; p.K = s.K; p.OH = plan->OH; p.OW = plan->OW; p.relu = relu;
-    p.tH = plan->tiles_h; p.tW = plan->tiles_w; p.tileN = p.tH * p.tW;
-    p.K_pad = plan->K_pad; p.T_pad = plan->T_pad;
-    int best = 0, bestP = 0, bestR = 0;
-    double bestUtil = -1.0;
-    const int cand[3] = {64, 128, 256};
-    for (int i = 0; i < 3; i++) {
-        int P, R;
-        if (!chunking(cand[i], s.N, p.tH, p.tW, &P, &R)) continue;
-        const int nBG = (p.tH + R - 1) / R;
-        const double util = (double)p.tH * p.tW * P / ((double)nBG * cand[i]);
-        if (util > bestUtil + 0.02) { bestUtil = util; best = cand[i]; bestP = P; bestR = R; }
-    }
-    if (!best) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_output_transform: image too wide", hipSuccess);
-    p.P = bestP; p.R = bestR;
-    p.nPG = (s.N + p.P - 1) / p.P;
-    p.nBG = (p.tH + p.R - 1) / p.R;
-    p.divR = fc_make_fastdiv(p.R);
+    p.tH = plan->tiles_h; p.tW = plan->tiles_w;
+    p.T = plan->T; p.K_pad = plan->K_pad; p.T_pad = plan->T_pad;
+    p.divTH = fc_make_fastdiv(p.tH);
     p.divTW = fc_make_fastdiv(p.tW);
-    const size_t ldsBytes = (size_t)p.P * min(p.R * 6, p.OH) * p.OW * sizeof(float);
-    const dim3 grid(p.nPG * p.nBG, s.K);
+    const int tpb = (plan->T_pad % 128 == 0 && plan->T >= 128) ? 128 : 64;
+    const int maxBands = (tpb + p.tW - 2) / p.tW + 1;
+    const size_t ldsBytes = (size_t)maxBands * 6 * p.OW * sizeof(float);
+    if (ldsBytes > 64 * 1024) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_output_transform: image too wide", hipSuccess);
+    const dim3 grid((unsigned)((plan->T + tpb - 1) / tpb), s.K);
     if (grid.y > 65535) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_output_transform: more than 65535 channels", hipSuccess);
+    if (((uintptr_t)y_dev & 15) != 0) return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_output_transform: y must be 16-byte aligned", hipSuccess);
     fc_stage_scope scope(ctx, FC_STAGE_OUTPUT_TRAN);
-    if (best == 64) wino_output_transform_kernel<64><<<grid, dim3(64), ldsBytes, ctx->stream>>>(p);
-    else if (best == 128) wino_output_transform_kernel<128><<<grid, dim3(128), ldsBytes, ctx->stream>>>(p);
-    else wino_output_transform_kernel<256><<<grid, dim3(256), ldsBytes, ctx->stream>>>(p);
+    if (tpb == 128) wino_output_transform_kernel<128><<<grid, dim3(128), ldsBytes, ctx->stream>>>(p);
+    else wino_output_transform_kernel<64><<<grid, dim3(64), ldsBytes, ctx->stream>>>(p);
     FC_LAUNCH_CHECK(ctx, "wino_output_transform_kernel");
     return FC_OK;
 }
