@@ -131,6 +131,27 @@ def cpu_baseline(target_seconds=12.0):
                       % (batch, s1)}
 
 
+def copy_probe(mib):
+    """Plain device-to-device copy of a known size: what FETCH_SIZE / WRITE_SIZE read for it is
+    the factor the counters of the other kernels are scaled by."""
+    import fastconv_amd as F
+    nbytes = mib << 20
+    L = F.load(0, 2 * nbytes + (64 << 20))
+    src, dst = L.alloc(nbytes), L.alloc(nbytes)
+    L.fill_zero(src, nbytes)
+    L.device_copy(dst, src, nbytes)
+    L.sync()
+    t0 = time.perf_counter()
+    reps = 5
+    for _ in range(reps):
+        L.device_copy(dst, src, nbytes)
+    L.sync()
+    dt = (time.perf_counter() - t0) / reps
+    print(json.dumps({"probe": "copy", "bytes_read": nbytes, "bytes_written": nbytes, "launches": reps + 1,
+                      "ms": round(dt * 1e3, 4), "GBps_read_plus_write": round(2 * nbytes / dt / 1e9, 1)}), flush=True)
+    L.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -143,7 +164,14 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--stage-events", default="all", choices=["all", "gemm", "none"],
                     help="which kernels are bracketed by events inside the timed region")
+    ap.add_argument("--timed-only", action="store_true",
+                    help="no per-layer detail pass after the timed region (every launch of the process is then a "
+                         "warm-up or timed step: what a kernel trace of this command averages over)")
+    ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
+                    help="only run the plain copy kernel over MIB mebibytes (scale for the HBM traffic counters)")
     args = ap.parse_args()
+    if args.copy_probe:
+        return copy_probe(args.copy_probe)
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the layers shard by batch with no exchange step; "
               "see DESIGN.md); run with --gpus 1", file=sys.stderr)
@@ -169,11 +197,7 @@ def main():
     # tile shape per layer
     for lay in layers:
         if args.no_tune:
-            cfg, ms = 0, 0.0
-            for c in L.wino_configs():     # first configuration that does not over-pad K
-                if L.wino_plan(lay.shape, c.id).K_pad < 2 * lay.K or c.bm == 32:
-                    cfg = c.id
-                    break
+            cfg, ms = L.wino_default_config(lay.shape), 0.0      # the library's untuned choice
         else:
             cfg, ms = tune_layer(L, lay, V, M, (vmax, mmax))
         lay.plan = L.wino_plan(lay.shape, cfg)
@@ -233,7 +257,7 @@ def main():
     # per-layer detail, outside the timed region
     per_layer = []
     L.timing(0x0f)
-    for lay in layers:
+    for lay in ([] if args.timed_only else layers):
         L.timing_reset()
         reps = 5
         t0 = time.perf_counter()

@@ -74,11 +74,14 @@ _ABI = {
     "fc_upload": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
     "fc_download": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
     "fc_fill_zero": (C.c_int, [_vp, _vp, C.c_size_t]),
+    "fc_device_copy": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
     "fc_timing_enable": (C.c_int, [_vp, C.c_int]),
     "fc_timing_reset": (C.c_int, [_vp]),
     "fc_stage_time_ms": (C.c_int, [_vp, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_long)]),
     "fc_wino_gemm_num_configs": (C.c_int, []),
     "fc_wino_gemm_get_config": (C.c_int, [C.c_int, C.POINTER(GemmConfig)]),
+    "fc_wino_gemm_default_config": (C.c_int, [C.POINTER(ConvShape)]),
+    "fc_igemm_default_config": (C.c_int, [C.POINTER(ConvShape)]),
     "fc_wino_make_plan": (C.c_int, [C.POINTER(ConvShape), C.c_int, C.POINTER(WinoPlan)]),
     "fc_wino_filter_transform": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp]),
     "fc_wino_input_transform": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp]),
@@ -184,6 +187,9 @@ class Library:
     def fill_zero(self, ptr, nbytes):
         self._check(self.c.fc_fill_zero(self.ctx, ptr, nbytes))
 
+    def device_copy(self, dst, src, nbytes):
+        self._check(self.c.fc_device_copy(self.ctx, dst, src, nbytes))
+
     def sync(self):
         self._check(self.c.fc_sync(self.ctx))
 
@@ -226,6 +232,12 @@ class Library:
             out.append(g)
         return out
 
+    def wino_default_config(self, shape):
+        return self.c.fc_wino_gemm_default_config(C.byref(shape))
+
+    def igemm_default_config(self, shape):
+        return self.c.fc_igemm_default_config(C.byref(shape))
+
     def wino_plan(self, shape, config=0):
         plan = WinoPlan()
         rc = self.c.fc_wino_make_plan(C.byref(shape), config, C.byref(plan))
@@ -265,8 +277,8 @@ class Library:
         self._check(self.c.fc_conv_implicit_gemm(self.ctx, C.byref(plan), x, Wp, table, bias, int(relu), y))
 
     # ---- whole-layer helpers over host arrays (tests, smoke)
-    def winograd_conv(self, shape, x, w, bias=None, relu=False, config=0, stages=False):
-        plan = self.wino_plan(shape, config)
+    def winograd_conv(self, shape, x, w, bias=None, relu=False, config=None, stages=False):
+        plan = self.wino_plan(shape, self.wino_default_config(shape) if config is None else config)
         mark = C.c_size_t()
         self._check(self.c.fc_pool_mark(self.pool, C.byref(mark)))
         try:
@@ -285,8 +297,8 @@ class Library:
         finally:
             self._check(self.c.fc_pool_release(self.pool, mark.value))
 
-    def implicit_gemm_conv(self, shape, x, w, bias=None, relu=False, config=0):
-        plan = self.igemm_plan(shape, config)
+    def implicit_gemm_conv(self, shape, x, w, bias=None, relu=False, config=None):
+        plan = self.igemm_plan(shape, self.igemm_default_config(shape) if config is None else config)
         mark = C.c_size_t()
         self._check(self.c.fc_pool_mark(self.pool, C.byref(mark)))
         try:

@@ -225,6 +225,23 @@ extern "C" int fc_fill_zero(fc_context *ctx, void *dst_dev, size_t bytes) {
     return FC_OK;
 }
 
+__global__ __launch_bounds__(256) void fc_copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[i] = src[i];
+}
+
+extern "C" int fc_device_copy(fc_context *ctx, void *dst_dev, const void *src_dev, size_t bytes) {
+    if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    if (!dst_dev || !src_dev || (bytes & 15) || (((uintptr_t)dst_dev | (uintptr_t)src_dev) & 15))
+        return fc_set_error(ctx, FC_ERR_INVALID, "fc_device_copy: pointers and size must be 16-byte multiples", hipSuccess);
+    if (bytes == 0) return FC_OK;
+    const size_t n = bytes / 16, blocks = (n + 255) / 256;
+    if (blocks >= (1ull << 31)) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_device_copy: more than 512 GiB", hipSuccess);
+    fc_copy_kernel<<<dim3((unsigned)blocks), dim3(256), 0, ctx->stream>>>((const uint4 *)src_dev, (uint4 *)dst_dev, n);
+    FC_LAUNCH_CHECK(ctx, "fc_copy_kernel");
+    return FC_OK;
+}
+
 // --------------------------------------------------------------- timing
 
 static int fc_timing_fold(fc_context *ctx) {

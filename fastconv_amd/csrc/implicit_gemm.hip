@@ -5,6 +5,8 @@
 // it straight into LDS.  The filter is re-laid once to Wp[Kred_pad][K_pad]
 // (output channel fastest) so that its tiles are straight 16-byte copies, as in
 // the Winograd GEMM.
+#include <cmath>
+
 #include "fc_internal.h"
 
 namespace {
@@ -215,6 +217,27 @@ extern "C" int fc_igemm_get_config(int id, fc_gemm_config *cfg) {
     if (!cfg || id < 0 || id >= kNumIgConfigs) return FC_ERR_INVALID;
     *cfg = kIgConfigs[id];
     return FC_OK;
+}
+
+extern "C" int fc_igemm_default_config(const fc_conv_shape *s) {
+    if (!fc_shape_ok(s)) return FC_ERR_INVALID;
+    const double M = s->K, Kr = (double)s->C * s->kh * s->kw;
+    const double Np = (double)s->N * fc_out_dim(s->H, s->pt, s->pb, s->kh, s->sh) * fc_out_dim(s->W, s->pl, s->pr, s->kw, s->sw);
+    int best = 0;
+    double bestCost = 1e300;
+    for (int id = 0; id < kNumIgConfigs; id++) {
+        const fc_gemm_config &c = kIgConfigs[id];
+        const double mp = ceil(M / c.bm) * c.bm, np = ceil(Np / c.bn) * c.bn, kp = ceil(Kr / c.bk) * c.bk;
+        double eff = (128.0 + 128.0) / (128.0 * 128.0) / ((double)(c.bm + c.bn) / ((double)c.bm * c.bn));
+        if (eff > 1.0) eff = 1.0;
+        if (c.bm * c.bn > 128 * 128) eff *= 0.8;       // one resident workgroup per SIMD set
+        const double blocks = (mp / c.bm) * (np / c.bn);
+        const double slots = 256.0 * (c.bm * c.bn > 128 * 128 ? 1 : 3);
+        const double fill = blocks / (ceil(blocks / slots) * slots);
+        const double cost = mp * np * kp / (eff * (0.25 + 0.75 * fill));
+        if (cost < bestCost) { bestCost = cost; best = id; }
+    }
+    return best;
 }
 
 extern "C" int fc_igemm_make_plan(const fc_conv_shape *s, int config, fc_igemm_plan *plan) {

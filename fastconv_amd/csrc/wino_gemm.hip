@@ -4,6 +4,7 @@
 // fastest, which is exactly the order v_mfma_f32_32x32x2_f32 wants its lanes in
 // (lane l holds row/col l%32 of reduction step l/32), so tiles go global -> LDS
 // as straight 16-byte copies and LDS -> registers as conflict-free dword reads.
+#include <cmath>
 #include <utility>
 
 #include "fc_internal.h"
@@ -198,6 +199,33 @@ extern "C" int fc_wino_gemm_get_config(int id, fc_gemm_config *cfg) {
     if (!cfg || id < 0 || id >= kNumConfigs) return FC_ERR_INVALID;
     *cfg = kConfigs[id];
     return FC_OK;
+}
+
+// Cost model behind the untuned choice: padded multiply-adds, divided by a relative
+// rate per tile shape (operand traffic per flop grows as (bm+bn)/(bm*bn); measured
+// on MI355X the 128x128 tile sustains the highest rate) and by how evenly the grid
+// fills the 256 CUs x 4 resident workgroups.
+extern "C" int fc_wino_gemm_default_config(const fc_conv_shape *s) {
+    if (!fc_shape_ok(s)) return FC_ERR_INVALID;
+    const int OH = fc_out_dim(s->H, s->pt, s->pb, 3, 1), OW = fc_out_dim(s->W, s->pl, s->pr, 3, 1);
+    const double T = (double)s->N * ((OH + 5) / 6) * ((OW + 5) / 6);
+    int best = 0;
+    double bestCost = 1e300;
+    for (int id = 0; id < kNumConfigs; id++) {
+        const fc_gemm_config &c = kConfigs[id];
+        const double kp = ceil((double)s->K / c.bm) * c.bm, tp = ceil(T / c.bn) * c.bn;
+        const double cp = ceil((double)s->C / c.bk) * c.bk;
+        double eff = (128.0 + 128.0) / (128.0 * 128.0) / ((double)(c.bm + c.bn) / ((double)c.bm * c.bn));
+        if (eff > 1.0) eff = 1.0;
+        if (c.bm * c.bn > 128 * 128) eff *= 0.93;      // 2 resident workgroups per CU instead of 4
+        if (c.bk == 32) eff *= 0.95;
+        const double blocks = 64.0 * (kp / c.bm) * (tp / c.bn);
+        const double slots = 256.0 * (c.bm * c.bn > 128 * 128 ? 2 : 4);
+        const double fill = blocks / (ceil(blocks / slots) * slots);
+        const double cost = kp * tp * cp / (eff * (0.4 + 0.6 * fill));
+        if (cost < bestCost) { bestCost = cost; best = id; }
+    }
+    return best;
 }
 
 extern "C" int fc_wino_gemm(fc_context *ctx, const fc_wino_plan *plan, const float *U_dev, const float *V_dev,

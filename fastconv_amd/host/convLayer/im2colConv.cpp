@@ -1,8 +1,5 @@
 #include "im2colConv.h"
 
-#include <float.h>
-#include <math.h>
-
 #include "../utility/tuning_log.h"
 
 using fastconv::Device;
@@ -21,32 +18,16 @@ ConvIm2colLayer::ConvIm2colLayer(float *input, float *kernel, float *biasw, floa
     channel_bias = NULL;
     relu = false;
     if (bias) fprintf(stderr, "Warning: the per-element bias tensor is ignored by the im2col layer (use SetChannelBias)\n");
-    config_best = (tile_config >= 0 && tile_config < fc_igemm_num_configs()) ? tile_config : DefaultConfig(M, N, K);
+    config_best = tile_config;
+    if (config_best < 0 || config_best >= fc_igemm_num_configs()) {
+        const fc_conv_shape s = Shape();
+        config_best = fc_igemm_default_config(&s);
+        if (config_best < 0) config_best = 0;
+    }
     config = config_best;
 }
 
 ConvIm2colLayer::~ConvIm2colLayer() { dev.Release(); }
-
-// Tile shape used without tuning: least padded work, discounted for small tiles
-// (more operand traffic per flop) and for grids that leave CUs idle.
-int ConvIm2colLayer::DefaultConfig(int M, long N, int K) {
-    int best = 0;
-    double bestCost = DBL_MAX;
-    for (int id = 0; id < fc_igemm_num_configs(); id++) {
-        fc_gemm_config c;
-        fc_igemm_get_config(id, &c);
-        const double mp = ceil((double)M / c.bm) * c.bm, np = ceil((double)N / c.bn) * c.bn;
-        const double kp = ceil((double)K / c.bk) * c.bk;
-        double eff = (128.0 + 128.0) / (128.0 * 128.0) / ((double)(c.bm + c.bn) / ((double)c.bm * c.bn));
-        if (eff > 1.0) eff = 1.0;
-        const double blocks = (mp / c.bm) * (np / c.bn);
-        const double waves = ceil(blocks / 512.0);
-        const double fill = blocks / (waves * 512.0);
-        const double cost = mp * np * kp / (eff * (0.25 + 0.75 * fill));
-        if (cost < bestCost) { bestCost = cost; best = id; }
-    }
-    return best;
-}
 
 fc_conv_shape ConvIm2colLayer::Shape() const {
     fc_conv_shape s;

@@ -29,8 +29,6 @@ class ConvIm2colLayer : public ConvLayer {
     int best_config() const { return config_best; }
     double gemm_ms = 0.0;   // per-Forward milliseconds of the implicit-GEMM kernel in the last Forward()
 
-    static int DefaultConfig(int M, long N, int K);
-
    protected:
     int M;
     long N;

@@ -24,7 +24,7 @@ ConvWinoF63Layer::ConvWinoF63Layer(float *input, float *kernel, float *biasw, fl
     if (bias) fprintf(stderr, "Warning: the per-element bias tensor is ignored by the Winograd layer (use SetChannelBias)\n");
     const size_t tileN = ((output_height + 5) / 6) * ((output_width + 5) / 6);
     imgBlock_best = DefaultImagesPerBlock(oc, ic, tileN, n, kCacheBudget);
-    gemmConfig_best = ConvWinoF63ZCLayer::DefaultConfig(oc, ic, (long)imgBlock_best * tileN);
+    gemmConfig_best = ConvWinoF63ZCLayer::DefaultConfig(oc, ic, ih, iw, pad_top, imgBlock_best);
     enableOffKernel = 1;
     tileBlock = ocBlock = icBlock = ocRegBlock = tileRegBlock = imgBlock = 0;
 }

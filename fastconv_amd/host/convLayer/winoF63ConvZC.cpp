@@ -1,8 +1,5 @@
 #include "winoF63ConvZC.h"
 
-#include <float.h>
-#include <math.h>
-
 #include "../utility/tuning_log.h"
 
 using fastconv::Device;
@@ -21,8 +18,7 @@ ConvWinoF63ZCLayer::ConvWinoF63ZCLayer(float *input, float *kernel, float *biasw
         exit(EXIT_FAILURE);
     }
     if (bias) fprintf(stderr, "Warning: the per-element bias tensor is ignored by the Winograd layer (use SetChannelBias)\n");
-    const long T = (long)n * ((output_height + 5) / 6) * ((output_width + 5) / 6);
-    gemmConfig_best = DefaultConfig(oc, ic, T);
+    gemmConfig_best = DefaultConfig(oc, ic, ih, iw, pad_top, n);
     scheduling_best = 0;
     gemmConfig = gemmConfig_best;
     enableOffKernel = scheduling = 0;
@@ -31,29 +27,13 @@ ConvWinoF63ZCLayer::ConvWinoF63ZCLayer(float *input, float *kernel, float *biasw
 
 ConvWinoF63ZCLayer::~ConvWinoF63ZCLayer() { dev.Release(); }
 
-// Tile shape used without tuning: the candidate with the least padded work,
-// weighted by how well each shape keeps the MFMA pipe fed (measured on MI355X:
-// the 128x128 tile reaches the highest rate, narrower tiles proportionally less).
-int ConvWinoF63ZCLayer::DefaultConfig(size_t K, size_t C, long T) {
-    int best = 0;
-    double bestCost = DBL_MAX;
-    for (int id = 0; id < fc_wino_gemm_num_configs(); id++) {
-        fc_gemm_config c;
-        fc_wino_gemm_get_config(id, &c);
-        const double kp = ceil((double)K / c.bm) * c.bm, tp = ceil((double)T / c.bn) * c.bn;
-        const double cp = ceil((double)C / c.bk) * c.bk;
-        const double area = (double)c.bm * c.bn;
-        // rate relative to the 128x128 tile: operand traffic per flop grows as (bm+bn)/(bm*bn)
-        double eff = (128.0 + 128.0) / (128.0 * 128.0) / ((c.bm + c.bn) / area);
-        if (eff > 1.0) eff = 1.0;
-        if (c.bk != 16) eff *= 0.95;
-        const double blocks = 64.0 * (kp / c.bm) * (tp / c.bn);
-        const double waves = ceil(blocks / 512.0);          // 256 CUs x 2 workgroups in flight
-        const double fill = blocks / (waves * 512.0);
-        const double cost = kp * tp * cp / (eff * (0.5 + 0.5 * fill));
-        if (cost < bestCost) { bestCost = cost; best = id; }
-    }
-    return best;
+// Tile shape used without tuning: the library's cost model.
+int ConvWinoF63ZCLayer::DefaultConfig(size_t K, size_t C, size_t H, size_t W, size_t pad, size_t N) {
+    fc_conv_shape s;
+    s.N = (int)N; s.C = (int)C; s.H = (int)H; s.W = (int)W; s.K = (int)K;
+    s.kh = s.kw = 3; s.sh = s.sw = 1; s.pt = s.pb = s.pl = s.pr = (int)pad;
+    const int id = fc_wino_gemm_default_config(&s);
+    return id < 0 ? 0 : id;
 }
 
 fc_conv_shape ConvWinoF63ZCLayer::Shape() const {

@@ -37,7 +37,7 @@ class ConvWinoF63ZCLayer : public ConvLayer {
     // per-Forward milliseconds of the last Forward(): InputTran, KernelTran, TensorGEMM, OutputTran
     double stage_ms[4] = {0, 0, 0, 0};
 
-    static int DefaultConfig(size_t K, size_t C, long T);
+    static int DefaultConfig(size_t K, size_t C, size_t H, size_t W, size_t pad, size_t N);
 
    private:
     fc_conv_shape Shape() const;

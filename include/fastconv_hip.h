@@ -98,6 +98,10 @@ int fc_pool_stats(fc_pool *pool, size_t *capacity, size_t *used, size_t *peak);
 int fc_upload(fc_context *ctx, void *dst_dev, const void *src_host, size_t bytes);
 int fc_download(fc_context *ctx, void *dst_host, const void *src_dev, size_t bytes);
 int fc_fill_zero(fc_context *ctx, void *dst_dev, size_t bytes);
+/* Device-to-device copy by a plain kernel (16 bytes per lane): the known-size
+ * reference that hardware traffic counters are scaled by.  Both pointers and the
+ * size must be multiples of 16. */
+int fc_device_copy(fc_context *ctx, void *dst_dev, const void *src_dev, size_t bytes);
 
 /* ---- stage timing (utility/helper.h:66-80 Timer, per stage) ----------- */
 
@@ -127,6 +131,11 @@ typedef struct {
 
 int fc_wino_gemm_num_configs(void);
 int fc_wino_gemm_get_config(int id, fc_gemm_config *cfg);
+/* Tile shape to use when a layer has not been tuned (the role of the defaults
+ * ocBlock=140, tileBlock=52, icBlock=64 in convLayer/winoF63ConvZC.cpp:11-16):
+ * the shape with the least padded work, discounted for narrow tiles and for
+ * grids that leave compute units idle.  Returns a configuration id. */
+int fc_wino_gemm_default_config(const fc_conv_shape *shape);
 
 /* Buffer geometry for one layer under one GEMM configuration.  Frequencies
  * f = 8*row + col of the transformed 8x8 tile; tiles t = (n*tiles_h + th)*tiles_w + tw.
@@ -185,6 +194,9 @@ int fc_wino_forward(fc_context *ctx, const fc_wino_plan *plan, const float *x_de
 
 int fc_igemm_num_configs(void);
 int fc_igemm_get_config(int id, fc_gemm_config *cfg);
+/* Untuned choice, as above (the role of mc=8, nc=256, kc=384 in
+ * convLayer/im2colConv.h:17-18). */
+int fc_igemm_default_config(const fc_conv_shape *shape);
 
 /* Filter re-layout done once at Init: Wp[Kred_pad][K_pad], output channel
  * fastest, reduction index (c, r, s) as in the column matrix rows
