@@ -24,6 +24,10 @@ sys.path.insert(0, ROOT)
 
 PEAK_MFMA_F32_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch of the GEMM kernel (FETCH_SIZE + WRITE_SIZE, scaled by the copy kernel), averaged
+# over the 13 layer passes of the default workload; from profiles/vgg16_b32_winograd_hbm_traffic_pmc.txt.
+# The counters need their own rocprofv3 runs, so this is not re-measured by every bench run.
+MEASURED_GEMM_TRAFFIC = {"vgg16_b32": 485.7e6}
 
 # (C, K, H, repeats)
 VGG16 = [(3, 64, 224, 1), (64, 64, 224, 1), (64, 128, 112, 1), (128, 128, 112, 1), (128, 256, 56, 1),
@@ -241,6 +245,9 @@ def main():
     if stage[ST_GEMM][1] > 0:
         gemm_ms, gemm_cnt = stage[ST_GEMM]
         ach = gemm_flops_step * (gemm_cnt / launches_step) / (gemm_ms * 1e-3) / 1e12
+        roofline["traffic"] = MEASURED_GEMM_TRAFFIC.get(args.workload)
+        roofline["algorithmic_bytes_per_launch_avg"] = round(
+            sum(256.0 * (l.K * l.C + l.C * l.plan.T + l.K * l.plan.T) * l.repeats for l in layers) / launches_step)
         roofline.update(achieved=round(ach, 2), frac=round(ach / PEAK_MFMA_F32_TFLOPS, 4),
                         launches=gemm_cnt, avg_launch_ms=round(gemm_ms / gemm_cnt, 5),
                         flops_per_launch_avg=gemm_flops_step / launches_step)
