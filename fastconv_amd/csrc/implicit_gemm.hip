@@ -6,6 +6,7 @@
 // (output channel fastest) so that its tiles are straight 16-byte copies, as in
 // the Winograd GEMM.
 #include <cmath>
+#include <utility>
 
 #include "fc_internal.h"
 
@@ -16,7 +17,7 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));   // native vector: a
 
 // Row table entry for reduction index kred = (c*kh + r)*kw + s:
 //   [2*kred]   = c*H*W + r*W + s      (offset from the window origin)
-//   [2*kred+1] = r << 16 | s          (0x7fff7fff for padding rows: never in bounds)
+//   [2*kred+1] = r << 16 | s          (31 << 16 | 31 for padding rows: a mask bit that is never set)
 __global__ __launch_bounds__(256) void igemm_pack_filter_kernel(const float *__restrict__ w,
                                                                 float *__restrict__ Wp,
                                                                 int32_t *__restrict__ table, int K, int C,
@@ -33,7 +34,7 @@ __global__ __launch_bounds__(256) void igemm_pack_filter_kernel(const float *__r
             table[2 * kred + 1] = (r << 16) | s;
         } else {
             table[2 * kred] = 0;
-            table[2 * kred + 1] = 0x7fff7fff;
+            table[2 * kred + 1] = (31 << 16) | 31;
         }
     }
 }
@@ -44,7 +45,7 @@ struct IgemmParams {
     const int32_t *table;
     const float *bias;
     float *y;
-    int N, C, H, W, K, OH, OW, sh, sw, pt, pl, relu;
+    int N, C, H, W, K, OH, OW, kh, kw, sh, sw, pt, pl, relu;
     int Kred_pad, K_pad;
     long Npix;
     int nKB, nPB;
@@ -58,121 +59,157 @@ struct IgTile {
     static constexpr int WM = BM / WGM, WN = BN / WGN;
     static constexpr int MI = WM / 32, NI = WN / 32;
     static constexpr int A_VEC = BK * BM / 4;
-    static constexpr int A_LD = (A_VEC + THREADS - 1) / THREADS;
+    static constexpr int A_LD = A_VEC / THREADS;
+    static constexpr int A_ROWS = THREADS * 4 / BM;     // filter-tile rows per copy pass
     static constexpr int ROW_STEP = THREADS / BN;       // gather: one column, every ROW_STEP-th row
     static constexpr int B_LD = BK / ROW_STEP;
     static constexpr int LDS_BYTES = 2 * BK * (BM + BN) * 4;
     static_assert(THREADS % BN == 0 && BK % ROW_STEP == 0, "gather mapping");
+    static_assert(BN % 64 == 0, "a wavefront gathers one row of the column matrix");
+    static_assert(A_VEC % THREADS == 0 && A_LD >= 1, "every thread copies the same number of float4");
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be whole 32x32 MFMA blocks");
 };
+
+// Copy passes as pack expansions (literal register-array indices, see wino_gemm.hip).
+template <int... I>
+__device__ __forceinline__ void ig_load_rows(floatx4 (&r)[sizeof...(I)], const float *p, size_t rowStride,
+                                             std::integer_sequence<int, I...>) {
+    ((r[I] = *reinterpret_cast<const floatx4 *>(p + (size_t)I * rowStride)), ...);
+}
+template <int... I>
+__device__ __forceinline__ void ig_store_rows(float *lds, const floatx4 (&r)[sizeof...(I)], int rowStride,
+                                              std::integer_sequence<int, I...>) {
+    ((*reinterpret_cast<floatx4 *>(lds + I * rowStride) = r[I]), ...);
+}
+
+// One gathered element of the column matrix.  The row (reduction index) is the same
+// for the whole wavefront, so its table entry lives in scalar registers; the
+// per-pixel part of the bounds test is two bit masks computed once per thread.
+__device__ __forceinline__ float ig_gather(const float *ximg, int pixOff, uint32_t maskR, uint32_t maskS,
+                                           const int32_t *table, int kred) {
+    const int off = table[2 * kred], rs = table[2 * kred + 1];
+    const bool ok = ((maskR >> (rs >> 16)) & (maskS >> (rs & 0xffff)) & 1u) != 0;
+    const float v = ximg[ok ? pixOff + off : 0];      // always an in-bounds address
+    return ok ? v : 0.f;
+}
+template <int... I>
+__device__ __forceinline__ void ig_gather_rows(float (&r)[sizeof...(I)], const float *ximg, int pixOff,
+                                               uint32_t maskR, uint32_t maskS, const int32_t *table, int kred0,
+                                               int rowStep, std::integer_sequence<int, I...>) {
+    ((r[I] = ig_gather(ximg, pixOff, maskR, maskS, table, kred0 + I * rowStep)), ...);
+}
+template <int... I>
+__device__ __forceinline__ void ig_scatter_rows(float *lds, const float (&r)[sizeof...(I)], int rowStride,
+                                                std::integer_sequence<int, I...>) {
+    ((lds[I * rowStride] = r[I]), ...);
+}
 
 template <class TL>
 __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmParams p) {
     constexpr int BM = TL::BM_, BN = TL::BN_, BK = TL::BK_;
-    __shared__ __attribute__((aligned(16))) float As[2][BK][BM];
-    __shared__ __attribute__((aligned(16))) float Bs[2][BK][BN];
+    constexpr int MI = TL::MI, NI = TL::NI, A_LD = TL::A_LD, B_LD = TL::B_LD;
+    __shared__ __attribute__((aligned(16))) float As[2][BK * BM];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK * BN];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm0 = (wave / TL::WGN_) * TL::WM, wn0 = (wave % TL::WGN_) * TL::WN;
     // output-channel blocks innermost: neighbouring workgroups share the gathered pixels
     const int pb = blockIdx.x / p.nKB, kb = blockIdx.x - pb * p.nKB;
 
-    const float *Ag = p.Wp + (size_t)kb * BM;
+    // filter tile: straight 16-byte copies
+    const int arow = tid / (BM / 4), acol = (tid % (BM / 4)) * 4;
+    const float *ag = p.Wp + (size_t)arow * p.K_pad + (size_t)kb * BM + acol;
+    const size_t aStage = (size_t)BK * p.K_pad, aPass = (size_t)TL::A_ROWS * p.K_pad;
+    const int aLds = arow * BM + acol;
 
-    // the pixel column this thread gathers
-    const int gcol = tid % BN, grow0 = tid / BN;
+    // the pixel column this thread gathers; its wavefront shares the row
+    const int gcol = tid % BN;
+    const int grow0 = __builtin_amdgcn_readfirstlane(tid / BN);
     const long pix = (long)pb * BN + gcol;
-    const bool pixOK = pix < p.Npix;
-    int ih0 = 0, iw0 = 0;
-    const float *xwin = p.x;
-    if (pixOK) {
+    const float *ximg = p.x;
+    int pixOff = 0;
+    uint32_t maskR = 0, maskS = 0;
+    if (pix < p.Npix) {
         const uint32_t n = fc_div((uint32_t)pix, p.divOHW);
         const uint32_t pp = (uint32_t)pix - n * (uint32_t)(p.OH * p.OW);
         const uint32_t oh = fc_div(pp, p.divOW), ow = pp - oh * p.OW;
-        ih0 = (int)oh * p.sh - p.pt;
-        iw0 = (int)ow * p.sw - p.pl;
-        xwin = p.x + (size_t)n * p.C * p.H * p.W + (long)ih0 * p.W + iw0;
+        const int ih0 = (int)oh * p.sh - p.pt, iw0 = (int)ow * p.sw - p.pl;
+        ximg = p.x + (size_t)n * p.C * p.H * p.W;
+        pixOff = ih0 * p.W + iw0;
+        // bit r of maskR: row ih0 + r is inside the image (likewise maskS for columns)
+        for (int r = 0; r < p.kh; r++) maskR |= ((unsigned)(ih0 + r) < (unsigned)p.H) ? (1u << r) : 0u;
+        for (int q = 0; q < p.kw; q++) maskS |= ((unsigned)(iw0 + q) < (unsigned)p.W) ? (1u << q) : 0u;
     }
+    const int bLds = grow0 * BN + gcol;
 
-    floatx4 ra[TL::A_LD];
-    float rb[TL::B_LD];
+    using SeqA = std::make_integer_sequence<int, A_LD>;
+    using SeqB = std::make_integer_sequence<int, B_LD>;
+    floatx4 ra[A_LD];
+    float rb[B_LD];
+    ig_load_rows(ra, ag, aPass, SeqA());
+    ig_gather_rows(rb, ximg, pixOff, maskR, maskS, p.table, grow0, TL::ROW_STEP, SeqB());
 
-    auto load_global = [&](int k0) {
+    floatx16 acc[MI][NI];
 #pragma unroll
-        for (int i = 0; i < TL::A_LD; i++) {
-            const int v = tid + i * TL::THREADS;
-            if (TL::A_VEC % TL::THREADS == 0 || v < TL::A_VEC) {
-                const int row = v / (BM / 4), col = (v % (BM / 4)) * 4;
-                ra[i] = *reinterpret_cast<const floatx4 *>(Ag + (size_t)(k0 + row) * p.K_pad + col);
-            }
-        }
+    for (int mi = 0; mi < MI; mi++)
 #pragma unroll
-        for (int i = 0; i < TL::B_LD; i++) {
-            const int kred = k0 + grow0 + i * TL::ROW_STEP;
-            const int off = p.table[2 * kred], rs = p.table[2 * kred + 1];
-            const int ih = ih0 + (rs >> 16), iw = iw0 + (rs & 0xffff);
-            const bool ok = pixOK && (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
-            rb[i] = ok ? xwin[off] : 0.f;
-        }
-    };
-    auto store_lds = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < TL::A_LD; i++) {
-            const int v = tid + i * TL::THREADS;
-            if (TL::A_VEC % TL::THREADS == 0 || v < TL::A_VEC) {
-                const int row = v / (BM / 4), col = (v % (BM / 4)) * 4;
-                *reinterpret_cast<floatx4 *>(&As[buf][row][col]) = ra[i];
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < TL::B_LD; i++) Bs[buf][grow0 + i * TL::ROW_STEP][gcol] = rb[i];
-    };
-
-    floatx16 acc[TL::MI][TL::NI];
-#pragma unroll
-    for (int mi = 0; mi < TL::MI; mi++)
-#pragma unroll
-        for (int ni = 0; ni < TL::NI; ni++)
+        for (int ni = 0; ni < NI; ni++)
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[mi][ni][i] = 0.f;
 
-    load_global(0);
-    store_lds(0);
+    ig_store_rows(&As[0][aLds], ra, TL::A_ROWS * BM, SeqA());
+    ig_scatter_rows(&Bs[0][bLds], rb, TL::ROW_STEP * BN, SeqB());
     __syncthreads();
 
     const int lrow = lane >> 5, lcol = lane & 31;
+    const int aFrag = lrow * BM + wm0 + lcol, bFrag = lrow * BN + wn0 + lcol;
     const int nStages = p.Kred_pad / BK;
     for (int s = 0; s < nStages; s++) {
-        const int cur = s & 1;
-        if (s + 1 < nStages) load_global((s + 1) * BK);
+        const float *as = As[s & 1], *bs = Bs[s & 1];
+        const bool more = s + 1 < nStages;
+        if (more) {
+            ag += aStage;
+            ig_load_rows(ra, ag, aPass, SeqA());
+            ig_gather_rows(rb, ximg, pixOff, maskR, maskS, p.table, (s + 1) * BK + grow0, TL::ROW_STEP, SeqB());
+        }
+        float a[2][MI], bb[2][NI];
+#pragma unroll
+        for (int mi = 0; mi < MI; mi++) a[0][mi] = as[aFrag + mi * 32];
+#pragma unroll
+        for (int ni = 0; ni < NI; ni++) bb[0][ni] = bs[bFrag + ni * 32];
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 2) {
-            float a[TL::MI], bb[TL::NI];
+            const int cur = (kk >> 1) & 1, nxt = cur ^ 1;
+            if (kk + 2 < BK) {
 #pragma unroll
-            for (int mi = 0; mi < TL::MI; mi++) a[mi] = As[cur][kk + lrow][wm0 + mi * 32 + lcol];
+                for (int mi = 0; mi < MI; mi++) a[nxt][mi] = as[aFrag + (kk + 2) * BM + mi * 32];
 #pragma unroll
-            for (int ni = 0; ni < TL::NI; ni++) bb[ni] = Bs[cur][kk + lrow][wn0 + ni * 32 + lcol];
+                for (int ni = 0; ni < NI; ni++) bb[nxt][ni] = bs[bFrag + (kk + 2) * BN + ni * 32];
+            }
 #pragma unroll
-            for (int mi = 0; mi < TL::MI; mi++)
+            for (int mi = 0; mi < MI; mi++)
 #pragma unroll
-                for (int ni = 0; ni < TL::NI; ni++)
-                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[mi], bb[ni], acc[mi][ni], 0, 0, 0);
+                for (int ni = 0; ni < NI; ni++)
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][mi], bb[cur][ni], acc[mi][ni], 0, 0, 0);
         }
-        if (s + 1 < nStages) store_lds(cur ^ 1);
+        if (more) {
+            ig_store_rows(&As[(s & 1) ^ 1][aLds], ra, TL::A_ROWS * BM, SeqA());
+            ig_scatter_rows(&Bs[(s & 1) ^ 1][bLds], rb, TL::ROW_STEP * BN, SeqB());
+        }
         __syncthreads();
     }
 
     // epilogue: column = pixel (lane%32), rows = output channels
     const int OHW = p.OH * p.OW;
 #pragma unroll
-    for (int ni = 0; ni < TL::NI; ni++) {
+    for (int ni = 0; ni < NI; ni++) {
         const long opix = (long)pb * BN + wn0 + ni * 32 + lcol;
         if (opix >= p.Npix) continue;
         const uint32_t n = fc_div((uint32_t)opix, p.divOHW);
         const uint32_t pp = (uint32_t)opix - n * (uint32_t)OHW;
         float *yn = p.y + (size_t)n * p.K * OHW + pp;
 #pragma unroll
-        for (int mi = 0; mi < TL::MI; mi++)
+        for (int mi = 0; mi < MI; mi++)
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 const int k = kb * BM + wm0 + mi * 32 + 8 * (i / 4) + 4 * lrow + (i % 4);
@@ -245,7 +282,7 @@ extern "C" int fc_igemm_make_plan(const fc_conv_shape *s, int config, fc_igemm_p
     fc_gemm_config cfg;
     const int rc = fc_igemm_get_config(config, &cfg);
     if (rc) return rc;
-    if (s->kh > 0x7ffe || s->kw > 0x7ffe) return FC_ERR_UNSUPPORTED;
+    if (s->kh > 31 || s->kw > 31) return FC_ERR_UNSUPPORTED;      // the in-image test is a 32-bit mask per axis
     plan->shape = *s;
     plan->OH = fc_out_dim(s->H, s->pt, s->pb, s->kh, s->sh);
     plan->OW = fc_out_dim(s->W, s->pl, s->pr, s->kw, s->sw);
@@ -302,7 +339,7 @@ extern "C" int fc_conv_implicit_gemm(fc_context *ctx, const fc_igemm_plan *plan,
     IgemmParams p;
     p.x = x_dev; p.Wp = Wp_dev; p.table = table_dev; p.bias = bias_dev; p.y = y_dev;
     p.N = s.N; p.C = s.C; p.H = s.H; p.W = s.W; p.K = s.K; p.OH = plan->OH; p.OW = plan->OW;
-    p.sh = s.sh; p.sw = s.sw; p.pt = s.pt; p.pl = s.pl; p.relu = relu;
+    p.kh = s.kh; p.kw = s.kw; p.sh = s.sh; p.sw = s.sw; p.pt = s.pt; p.pl = s.pl; p.relu = relu;
     p.Kred_pad = plan->Kred_pad; p.K_pad = plan->K_pad; p.Npix = plan->Npix;
     p.nKB = plan->K_pad / cfg.bm;
     p.nPB = (int)((plan->Npix + cfg.bn - 1) / cfg.bn);
