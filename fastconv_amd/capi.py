@@ -46,7 +46,8 @@ class WinoPlan(C.Structure):
 class IgemmPlan(C.Structure):
     _fields_ = [("shape", ConvShape), ("OH", C.c_int), ("OW", C.c_int), ("Kred", C.c_int),
                 ("Kred_pad", C.c_int), ("K_pad", C.c_int), ("Npix", C.c_long), ("config", C.c_int),
-                ("Wp_bytes", C.c_size_t), ("table_bytes", C.c_size_t)]
+                ("Wp_bytes", C.c_size_t), ("table_bytes", C.c_size_t), ("split_k", C.c_int),
+                ("ws_bytes", C.c_size_t)]
 
 
 class DeviceInfo(C.Structure):
@@ -93,7 +94,7 @@ _ABI = {
     "fc_igemm_get_config": (C.c_int, [C.c_int, C.POINTER(GemmConfig)]),
     "fc_igemm_make_plan": (C.c_int, [C.POINTER(ConvShape), C.c_int, C.POINTER(IgemmPlan)]),
     "fc_igemm_pack_filter": (C.c_int, [_vp, C.POINTER(IgemmPlan), _vp, _vp, _vp]),
-    "fc_conv_implicit_gemm": (C.c_int, [_vp, C.POINTER(IgemmPlan), _vp, _vp, _vp, _vp, C.c_int, _vp]),
+    "fc_conv_implicit_gemm": (C.c_int, [_vp, C.POINTER(IgemmPlan), _vp, _vp, _vp, _vp, C.c_int, _vp, _vp]),
 }
 
 
@@ -273,8 +274,8 @@ class Library:
     def igemm_pack_filter(self, plan, w, Wp, table):
         self._check(self.c.fc_igemm_pack_filter(self.ctx, C.byref(plan), w, Wp, table))
 
-    def conv_implicit_gemm(self, plan, x, Wp, table, y, bias=None, relu=False):
-        self._check(self.c.fc_conv_implicit_gemm(self.ctx, C.byref(plan), x, Wp, table, bias, int(relu), y))
+    def conv_implicit_gemm(self, plan, x, Wp, table, y, bias=None, relu=False, ws=None):
+        self._check(self.c.fc_conv_implicit_gemm(self.ctx, C.byref(plan), x, Wp, table, bias, int(relu), ws, y))
 
     # ---- whole-layer helpers over host arrays (tests, smoke)
     def winograd_conv(self, shape, x, w, bias=None, relu=False, config=None, stages=False):
@@ -306,8 +307,9 @@ class Library:
             db = self.upload(bias) if bias is not None else None
             Wp, tab = self.alloc(plan.Wp_bytes), self.alloc(plan.table_bytes)
             y = self.alloc(4 * shape.N * shape.K * plan.OH * plan.OW)
+            ws = self.alloc(plan.ws_bytes) if plan.ws_bytes else None
             self.igemm_pack_filter(plan, dw, Wp, tab)
-            self.conv_implicit_gemm(plan, dx, Wp, tab, y, db, relu)
+            self.conv_implicit_gemm(plan, dx, Wp, tab, y, db, relu, ws)
             return self.download(y, (shape.N, shape.K, plan.OH, plan.OW))
         finally:
             self._check(self.c.fc_pool_release(self.pool, mark.value))

@@ -49,6 +49,8 @@ struct IgemmParams {
     int Kred_pad, K_pad;
     long Npix;
     int nKB, nPB;
+    int splitK, stagesPerSplit;   // reduction split over blockIdx.y; partial sums go to ws
+    float *ws;                    // [splitK][K][Npix] when splitK > 1
     fc_fastdiv divOHW, divOW;
 };
 
@@ -146,8 +148,12 @@ __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmPara
     using SeqB = std::make_integer_sequence<int, B_LD>;
     floatx4 ra[A_LD];
     float rb[B_LD];
+    // this block's share of the reduction
+    const int nStagesAll = p.Kred_pad / BK;
+    const int sBegin = blockIdx.y * p.stagesPerSplit, sEnd = min(sBegin + p.stagesPerSplit, nStagesAll);
+    ag += (size_t)sBegin * aStage;
     ig_load_rows(ra, ag, aPass, SeqA());
-    ig_gather_rows(rb, ximg, pixOff, maskR, maskS, p.table, grow0, TL::ROW_STEP, SeqB());
+    ig_gather_rows(rb, ximg, pixOff, maskR, maskS, p.table, sBegin * BK + grow0, TL::ROW_STEP, SeqB());
 
     floatx16 acc[MI][NI];
 #pragma unroll
@@ -163,10 +169,10 @@ __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmPara
 
     const int lrow = lane >> 5, lcol = lane & 31;
     const int aFrag = lrow * BM + wm0 + lcol, bFrag = lrow * BN + wn0 + lcol;
-    const int nStages = p.Kred_pad / BK;
-    for (int s = 0; s < nStages; s++) {
-        const float *as = As[s & 1], *bs = Bs[s & 1];
-        const bool more = s + 1 < nStages;
+    for (int s = sBegin; s < sEnd; s++) {
+        const int buf = (s - sBegin) & 1;
+        const float *as = As[buf], *bs = Bs[buf];
+        const bool more = s + 1 < sEnd;
         if (more) {
             ag += aStage;
             ig_load_rows(ra, ag, aPass, SeqA());
@@ -193,14 +199,31 @@ __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmPara
                     acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][mi], bb[cur][ni], acc[mi][ni], 0, 0, 0);
         }
         if (more) {
-            ig_store_rows(&As[(s & 1) ^ 1][aLds], ra, TL::A_ROWS * BM, SeqA());
-            ig_scatter_rows(&Bs[(s & 1) ^ 1][bLds], rb, TL::ROW_STEP * BN, SeqB());
+            ig_store_rows(&As[buf ^ 1][aLds], ra, TL::A_ROWS * BM, SeqA());
+            ig_scatter_rows(&Bs[buf ^ 1][bLds], rb, TL::ROW_STEP * BN, SeqB());
         }
         __syncthreads();
     }
 
     // epilogue: column = pixel (lane%32), rows = output channels
     const int OHW = p.OH * p.OW;
+    if (p.splitK > 1) {
+        // partial sums, [split][k][pixel]; igemm_reduce_kernel adds them up in split order
+        float *wz = p.ws + (size_t)blockIdx.y * p.K * p.Npix;
+#pragma unroll
+        for (int ni = 0; ni < NI; ni++) {
+            const long opix = (long)pb * BN + wn0 + ni * 32 + lcol;
+            if (opix >= p.Npix) continue;
+#pragma unroll
+            for (int mi = 0; mi < MI; mi++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int k = kb * BM + wm0 + mi * 32 + 8 * (i / 4) + 4 * lrow + (i % 4);
+                    if (k < p.K) wz[(size_t)k * p.Npix + opix] = acc[mi][ni][i];
+                }
+        }
+        return;
+    }
 #pragma unroll
     for (int ni = 0; ni < NI; ni++) {
         const long opix = (long)pb * BN + wn0 + ni * 32 + lcol;
@@ -223,6 +246,24 @@ __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmPara
     }
 }
 
+// Sums the partial results of a split reduction in split order (so the result does
+// not depend on which workgroup finished first), adds bias, applies ReLU, writes NCHW.
+__global__ __launch_bounds__(256) void igemm_reduce_kernel(const float *__restrict__ ws, const float *__restrict__ bias,
+                                                           float *__restrict__ y, int K, long Npix, int OHW,
+                                                           int splitK, int relu, fc_fastdiv divOHW) {
+    const long pix = (long)blockIdx.x * 256 + threadIdx.x;
+    const int k = blockIdx.y;
+    if (pix >= Npix) return;
+    const size_t slab = (size_t)K * Npix;
+    const float *src = ws + (size_t)k * Npix + pix;
+    float v = src[0];
+    for (int z = 1; z < splitK; z++) v += src[(size_t)z * slab];
+    if (bias) v += bias[k];
+    if (relu) v = fmaxf(v, 0.f);
+    const uint32_t n = fc_div((uint32_t)pix, divOHW);
+    y[((size_t)n * K + k) * OHW + (pix - (long)n * OHW)] = v;
+}
+
 typedef IgTile<128, 128, 16, 2, 2> Ig0;
 typedef IgTile<64, 128, 16, 1, 2> Ig1;
 typedef IgTile<128, 64, 16, 2, 1> Ig2;
@@ -242,7 +283,7 @@ const int kNumIgConfigs = sizeof(kIgConfigs) / sizeof(kIgConfigs[0]);
 
 template <class TL>
 void launch(fc_context *ctx, IgemmParams &p) {
-    const dim3 grid((unsigned)(p.nKB * p.nPB));
+    const dim3 grid((unsigned)(p.nKB * p.nPB), (unsigned)p.splitK);
     igemm_conv_kernel<TL><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
 }
 
@@ -296,6 +337,20 @@ extern "C" int fc_igemm_make_plan(const fc_conv_shape *s, int config, fc_igemm_p
     plan->config = config;
     plan->Wp_bytes = sizeof(float) * (size_t)plan->Kred_pad * plan->K_pad;
     plan->table_bytes = sizeof(int32_t) * 2 * (size_t)plan->Kred_pad;
+    // Small layers do not fill 256 CUs with (K_pad/BM) x (Npix/BN) workgroups: split the
+    // reduction until about three workgroups per CU exist, keeping >= 4 LDS stages per part.
+    const long blocks = (long)(plan->K_pad / cfg.bm) * ((npix + cfg.bn - 1) / cfg.bn);
+    const int stages = plan->Kred_pad / cfg.bk;
+    int split = 1;
+    if (blocks < 512) {
+        split = (int)((768 + blocks - 1) / blocks);
+        if (split > stages / 4) split = stages / 4;
+        if (split > 32) split = 32;
+        if (split < 1) split = 1;
+    }
+    const int per = (stages + split - 1) / split;
+    plan->split_k = (stages + per - 1) / per;          // no empty parts
+    plan->ws_bytes = plan->split_k > 1 ? sizeof(float) * (size_t)plan->split_k * s->K * npix : 0;
     return FC_OK;
 }
 
@@ -305,7 +360,8 @@ static int ig_plan_check(fc_context *ctx, const fc_igemm_plan *plan) {
     fc_igemm_plan chk;
     const int rc = fc_igemm_make_plan(&plan->shape, plan->config, &chk);
     if (rc) return fc_set_error(ctx, rc, "plan does not describe a supported layer", hipSuccess);
-    if (chk.Kred_pad != plan->Kred_pad || chk.K_pad != plan->K_pad || chk.Npix != plan->Npix)
+    if (chk.Kred_pad != plan->Kred_pad || chk.K_pad != plan->K_pad || chk.Npix != plan->Npix ||
+        chk.split_k != plan->split_k || chk.ws_bytes != plan->ws_bytes)
         return fc_set_error(ctx, FC_ERR_INVALID, "plan fields were modified after fc_igemm_make_plan", hipSuccess);
     return FC_OK;
 }
@@ -327,12 +383,14 @@ extern "C" int fc_igemm_pack_filter(fc_context *ctx, const fc_igemm_plan *plan, 
 
 extern "C" int fc_conv_implicit_gemm(fc_context *ctx, const fc_igemm_plan *plan, const float *x_dev,
                                      const float *Wp_dev, const int32_t *table_dev, const float *bias_dev, int relu,
-                                     float *y_dev) {
+                                     float *ws_dev, float *y_dev) {
     const int rc = ig_plan_check(ctx, plan);
     if (rc) return rc;
     if (!x_dev || !Wp_dev || !table_dev || !y_dev)
         return fc_set_error(ctx, FC_ERR_INVALID, "fc_conv_implicit_gemm: null buffer", hipSuccess);
     if ((uintptr_t)Wp_dev & 15) return fc_set_error(ctx, FC_ERR_INVALID, "fc_conv_implicit_gemm: Wp must be 16-byte aligned", hipSuccess);
+    if (plan->split_k > 1 && !ws_dev)
+        return fc_set_error(ctx, FC_ERR_INVALID, "fc_conv_implicit_gemm: this plan splits the reduction and needs ws_bytes of workspace", hipSuccess);
     fc_gemm_config cfg;
     fc_igemm_get_config(plan->config, &cfg);
     const fc_conv_shape &s = plan->shape;
@@ -345,6 +403,9 @@ extern "C" int fc_conv_implicit_gemm(fc_context *ctx, const fc_igemm_plan *plan,
     p.nPB = (int)((plan->Npix + cfg.bn - 1) / cfg.bn);
     p.divOHW = fc_make_fastdiv((uint32_t)(plan->OH * plan->OW));
     p.divOW = fc_make_fastdiv((uint32_t)plan->OW);
+    p.splitK = plan->split_k;
+    p.stagesPerSplit = ((plan->Kred_pad / cfg.bk) + plan->split_k - 1) / plan->split_k;
+    p.ws = ws_dev;
     if ((long)p.nKB * p.nPB >= (1l << 31)) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_conv_implicit_gemm: grid too large", hipSuccess);
     fc_stage_scope scope(ctx, FC_STAGE_IMPLICIT_GEMM);
     switch (plan->config) {
@@ -359,5 +420,12 @@ extern "C" int fc_conv_implicit_gemm(fc_context *ctx, const fc_igemm_plan *plan,
         default: return fc_set_error(ctx, FC_ERR_INVALID, "fc_conv_implicit_gemm: unknown tile configuration", hipSuccess);
     }
     FC_LAUNCH_CHECK(ctx, "igemm_conv_kernel");
+    if (plan->split_k > 1) {
+        const dim3 rgrid((unsigned)((plan->Npix + 255) / 256), (unsigned)s.K);
+        if (rgrid.y > 65535) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_conv_implicit_gemm: more than 65535 channels", hipSuccess);
+        igemm_reduce_kernel<<<rgrid, dim3(256), 0, ctx->stream>>>(ws_dev, bias_dev, y_dev, s.K, plan->Npix,
+                                                                  plan->OH * plan->OW, plan->split_k, relu, p.divOHW);
+        FC_LAUNCH_CHECK(ctx, "igemm_reduce_kernel");
+    }
     return FC_OK;
 }

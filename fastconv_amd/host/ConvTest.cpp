@@ -326,7 +326,8 @@ int main(int argc, char *argv[]) {
         if (options.algorithm == nnp_convolution_algorithm_winograd)
             bytes += 4 * 64 * (cpad * kpad + cpad * tpad + kpad * tpad);
         else
-            bytes += 4 * ((k_elems / output_channels + 32) * kpad) + 8 * (k_elems / output_channels + 32);
+            bytes += 4 * ((k_elems / output_channels + 32) * kpad) + 8 * (k_elems / output_channels + 32) +
+                     std::min<size_t>(32 * 4 * out_elems, (size_t)1 << 30);   // split-reduction workspace of small layers
         fastconv::Device::Configure(bytes);
     }
 

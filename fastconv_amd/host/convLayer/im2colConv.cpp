@@ -15,6 +15,7 @@ ConvIm2colLayer::ConvIm2colLayer(float *input, float *kernel, float *biasw, floa
     this->K = (int)(input_channels * kernel_height * kernel_width);
     packed_kernel = NULL;
     gather_table = NULL;
+    workspace = NULL;
     channel_bias = NULL;
     relu = false;
     if (bias) fprintf(stderr, "Warning: the per-element bias tensor is ignored by the im2col layer (use SetChannelBias)\n");
@@ -56,13 +57,14 @@ void ConvIm2colLayer::AllocateFor(int cfg) {
     config = cfg;
     packed_kernel = (float *)d.Alloc(plan.Wp_bytes, "packed kernel");
     gather_table = (int32_t *)d.Alloc(plan.table_bytes, "gather table");
+    workspace = plan.ws_bytes ? (float *)d.Alloc(plan.ws_bytes, "split-reduction workspace") : NULL;
     d.Check(fc_igemm_pack_filter(d.ctx(), &plan, dev.kernel, packed_kernel, gather_table), "fc_igemm_pack_filter");
 }
 
 void ConvIm2colLayer::RunOnce() {
     Device &d = Device::Get();
     d.Check(fc_conv_implicit_gemm(d.ctx(), &plan, dev.input, packed_kernel, gather_table, dev.bias, relu ? 1 : 0,
-                                  dev.output),
+                                  workspace, dev.output),
             "fc_conv_implicit_gemm");
 }
 
@@ -74,7 +76,8 @@ int ConvIm2colLayer::Init() {
     AllocateFor(config_best);
     fc_gemm_config c;
     fc_igemm_get_config(config, &c);
-    printf("Testing M=%d N=%ld K=%d batch=%zu tile %dx%dx%d (cfg %d)\n", M, N, K, batch, c.bm, c.bn, c.bk, config);
+    printf("Testing M=%d N=%ld K=%d batch=%zu tile %dx%dx%d (cfg %d) reduction split %d\n", M, N, K, batch, c.bm, c.bn,
+           c.bk, config, plan.split_k);
     return 1;
 }
 

@@ -42,6 +42,7 @@ class ConvIm2colLayer : public ConvLayer {
 
     float *packed_kernel;   // Wp[Kred_pad][K_pad], device
     int32_t *gather_table;  // device
+    float *workspace;       // device, partial sums when the plan splits the reduction
     fc_igemm_plan plan;
     LayerDeviceBuffers dev;
     const float *channel_bias;

@@ -208,6 +208,8 @@ typedef struct {
     long Npix;
     int config;
     size_t Wp_bytes, table_bytes;
+    int split_k;              /* > 1: the reduction is split over this many workgroups per tile */
+    size_t ws_bytes;          /* workspace for the partial sums ([split_k][K][Npix] floats), 0 if unsplit */
 } fc_igemm_plan;
 
 int fc_igemm_make_plan(const fc_conv_shape *shape, int config, fc_igemm_plan *plan);
@@ -219,10 +221,13 @@ int fc_igemm_pack_filter(fc_context *ctx, const fc_igemm_plan *plan, const float
 /* y[n][k][oh][ow] = sum_{c,r,s} w[k][c][r][s] * x[n][c][oh*sh+r-pt][ow*sw+s-pl].
  * Replaces ConvIm2colLayer::im2col_v1 + sgemm (convLayer/im2colConv.cpp:311-398,
  * 434-565) and the register kernels of im2col/gemm_kernel.cpp; the column matrix
- * is never materialised and y is overwritten (not accumulated). */
+ * is never materialised and y is overwritten (not accumulated).  Layers too small
+ * to fill the GPU have plan->split_k > 1: the reduction is cut into parts whose
+ * partial sums go to ws_dev (plan->ws_bytes) and are added in a fixed order by a
+ * second small kernel; ws_dev may be NULL when plan->ws_bytes is 0. */
 int fc_conv_implicit_gemm(fc_context *ctx, const fc_igemm_plan *plan, const float *x_dev,
                           const float *Wp_dev, const int32_t *table_dev,
-                          const float *bias_dev, int relu, float *y_dev);
+                          const float *bias_dev, int relu, float *ws_dev, float *y_dev);
 
 #ifdef __cplusplus
 }

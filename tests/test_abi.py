@@ -65,6 +65,12 @@ def test_plans_are_pure_host_arithmetic():
     assert lib.fc_igemm_make_plan(C.byref(s3), 0, C.byref(q)) == 0
     assert (q.OH, q.OW, q.Kred, q.Npix) == (4, 4, 27, 16)
     assert q.Kred_pad == 32 and q.K_pad == 128
+    assert q.split_k == 1 and q.ws_bytes == 0              # 2 stages: too short to split
+    # a batch-1 layer with 8 workgroups of output and a long reduction is split, with workspace
+    s4 = capi.ConvShape(1, 2048, 7, 7, 512, 1, 1, 1, 1, 0, 0, 0, 0)
+    assert lib.fc_igemm_make_plan(C.byref(s4), 0, C.byref(q)) == 0
+    assert q.split_k > 1 and q.ws_bytes == 4 * q.split_k * 512 * 49
+    assert (q.Kred_pad // 16) >= 4 * q.split_k
 
 
 def test_no_gpu_means_a_loud_error_not_a_fallback():

@@ -164,6 +164,24 @@ def test_implicit_gemm_every_tile_config(lib):
         assert O.max_rel_err(y, truth) <= TOL_IM2COL, cfg.id
 
 
+def test_implicit_gemm_split_reduction_is_exact_and_repeatable(lib):
+    """Batch-1 layers are too small to fill the GPU: their reduction is split and the parts
+    are added in a fixed order, so two runs give the same bits."""
+    for shp in [(1, 2048, 7, 7, 512, 1, 1, 1, 1, 0), (1, 256, 56, 56, 256, 3, 3, 1, 1, 1),
+                (1, 512, 14, 14, 512, 3, 3, 2, 2, 1), (1, 1024, 14, 14, 256, 1, 1, 1, 1, 0)]:
+        s = O.shape(*shp)
+        plan = lib.igemm_plan(cshape(s), lib.igemm_default_config(cshape(s)))
+        assert plan.split_k > 1, shp
+        x, w = O.make_inputs(s, seed=3)
+        bias = O.rng_uniform(9, (s.K,))
+        announce("split reduction", shp, "parts", plan.split_k)
+        y1 = lib.implicit_gemm_conv(cshape(s), x, w, bias=bias, relu=True)
+        y2 = lib.implicit_gemm_conv(cshape(s), x, w, bias=bias, relu=True)
+        assert np.array_equal(y1, y2)
+        truth = np.maximum(O.naive_conv_f64(s, x, w, bias), 0.0)
+        assert O.max_rel_err(y1, truth) <= TOL_IM2COL
+
+
 # ------------------------------------------- the reference's own naive layers
 
 def test_golden_vectors_of_reference_naive_layers(lib):
