@@ -66,6 +66,7 @@ class Layer:
         self.flops = self.shape.flops()
         self.plan = None
         self.U = None
+        self.fused = False
 
     def algorithmic(self):
         """Per-launch algorithmic work of each stage (flops for the GEMM, bytes for the transforms)."""
@@ -78,13 +79,17 @@ class Layer:
         }
 
 
-def forward(L, lay, V, M):
-    L.wino_forward(lay.plan, lay.x, lay.w, lay.U, V, M, lay.y)
+def forward(L, lay, V, M, filter_ready=False):
+    """One layer pass: staged (four kernels) or fused (GEMM + output transform in one kernel)."""
+    if lay.fused:
+        L.wino_forward_fused(lay.plan, lay.x, lay.w, lay.U, V, lay.y, filter_ready=filter_ready)
+    else:
+        L.wino_forward(lay.plan, lay.x, lay.w, lay.U, V, M, lay.y, filter_ready=filter_ready)
 
 
 def tune_layer(L, lay, V, M, scratch_bytes, iters=3):
     """Pick the GEMM tile shape with the shortest whole-layer forward."""
-    best = (None, 1e30)
+    best = (None, False, 1e30)
     for cfg in L.wino_configs():
         plan = L.wino_plan(lay.shape, cfg.id)
         if plan.V_bytes > scratch_bytes[0] or plan.M_bytes > scratch_bytes[1]:
@@ -94,16 +99,19 @@ def tune_layer(L, lay, V, M, scratch_bytes, iters=3):
         lay.plan = plan
         mark = L.mark()
         lay.U = L.alloc(plan.U_bytes)
-        forward(L, lay, V, M)
-        L.sync()
-        t0 = time.perf_counter()
-        for _ in range(iters):
+        # the fused kernel has one tile shape of its own; the plan only fixes the padding it reads
+        for fused in ((False, True) if lay.C * lay.K <= 16384 else (False,)):
+            lay.fused = fused
             forward(L, lay, V, M)
-        L.sync()
-        ms = (time.perf_counter() - t0) / iters * 1e3
+            L.sync()
+            t0 = time.perf_counter()
+            for _ in range(iters):
+                forward(L, lay, V, M)
+            L.sync()
+            ms = (time.perf_counter() - t0) / iters * 1e3
+            if ms < best[2]:
+                best = (cfg.id, fused, ms)
         L.release(mark)
-        if ms < best[1]:
-            best = (cfg.id, ms)
     return best
 
 
@@ -168,6 +176,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--stage-events", default="all", choices=["all", "gemm", "none"],
                     help="which kernels are bracketed by events inside the timed region")
+    ap.add_argument("--pipeline", default="auto", choices=["auto", "staged", "fused"],
+                    help="Winograd pipeline per layer: four staged kernels, GEMM + output transform fused, or "
+                         "whichever is faster for the layer (auto)")
     ap.add_argument("--timed-only", action="store_true",
                     help="no per-layer detail pass after the timed region (every launch of the process is then a "
                          "warm-up or timed step: what a kernel trace of this command averages over)")
@@ -200,15 +211,19 @@ def main():
 
     # tile shape per layer
     for lay in layers:
-        if args.no_tune:
-            cfg, ms = L.wino_default_config(lay.shape), 0.0      # the library's untuned choice
+        if args.no_tune:      # the library's untuned choices
+            cfg, fused, ms = L.wino_default_config(lay.shape), L.wino_prefer_fused(lay.shape), 0.0
         else:
-            cfg, ms = tune_layer(L, lay, V, M, (vmax, mmax))
+            cfg, fused, ms = tune_layer(L, lay, V, M, (vmax, mmax))
+        if args.pipeline != "auto":
+            fused = args.pipeline == "fused"
+        lay.fused = fused
         lay.plan = L.wino_plan(lay.shape, cfg)
         lay.U = L.alloc(lay.plan.U_bytes)
         L.wino_filter_transform(lay.plan, lay.w, lay.U)
         g = L.wino_configs()[cfg]
-        log("layer %d->%d @%d: tile %dx%dx%d (cfg %d) %.3f ms" % (lay.C, lay.K, lay.H, g.bm, g.bn, g.bk, cfg, ms))
+        log("layer %d->%d @%d: %s, tile %dx%dx%d (cfg %d) %.3f ms"
+            % (lay.C, lay.K, lay.H, "fused" if fused else "staged", g.bm, g.bn, g.bk, cfg, ms))
     L.sync()
 
     filter_ready = args.offline_filter
@@ -216,13 +231,13 @@ def main():
     def step():
         for lay in layers:
             for _ in range(lay.repeats):
-                L.wino_forward(lay.plan, lay.x, lay.w, lay.U, V, M, lay.y, filter_ready=filter_ready)
+                forward(L, lay, V, M, filter_ready)
 
     for _ in range(args.warmup):
         step()
     L.sync()
 
-    mask = {"all": 0x0f, "gemm": 1 << ST_GEMM, "none": 0}[args.stage_events]
+    mask = {"all": 0x4f, "gemm": 1 << ST_GEMM, "none": 0}[args.stage_events]
     L.timing(mask)
     L.timing_reset()
     t0 = time.perf_counter()
@@ -231,6 +246,7 @@ def main():
     L.sync()
     elapsed = time.perf_counter() - t0
     stage = [L.stage_time(i) for i in range(4)]
+    fused_stage = L.stage_time(6)
     L.timing(0)
 
     ms_per_step = elapsed / args.steps * 1e3
@@ -238,8 +254,9 @@ def main():
     value = step_flops / (ms_per_step * 1e-3) / 1e9
 
     # dominant kernel: the batched GEMM. achieved = algorithmic flops of all its launches / their event time
-    gemm_flops_step = sum(l.algorithmic()["gemm_flops"] * l.repeats for l in layers)
-    launches_step = sum(l.repeats for l in layers)
+    staged = [l for l in layers if not l.fused]
+    gemm_flops_step = sum(l.algorithmic()["gemm_flops"] * l.repeats for l in staged)
+    launches_step = max(1, sum(l.repeats for l in staged))
     roofline = {"kernel": "wino_gemm_kernel", "bound": "mfma", "achieved": None, "peak": PEAK_MFMA_F32_TFLOPS,
                 "unit": "TFLOP/s", "frac": None, "traffic": None}
     if stage[ST_GEMM][1] > 0:
@@ -247,23 +264,37 @@ def main():
         ach = gemm_flops_step * (gemm_cnt / launches_step) / (gemm_ms * 1e-3) / 1e12
         roofline["traffic"] = MEASURED_GEMM_TRAFFIC.get(args.workload)
         roofline["algorithmic_bytes_per_launch_avg"] = round(
-            sum(256.0 * (l.K * l.C + l.C * l.plan.T + l.K * l.plan.T) * l.repeats for l in layers) / launches_step)
+            sum(256.0 * (l.K * l.C + l.C * l.plan.T + l.K * l.plan.T) * l.repeats for l in staged) / launches_step)
         roofline.update(achieved=round(ach, 2), frac=round(ach / PEAK_MFMA_F32_TFLOPS, 4),
                         launches=gemm_cnt, avg_launch_ms=round(gemm_ms / gemm_cnt, 5),
                         flops_per_launch_avg=gemm_flops_step / launches_step)
     transforms = {}
+    all_launches = sum(l.repeats for l in layers)
     for name, idx, key in (("input_transform", ST_IT, "it_bytes"), ("output_transform", ST_OT, "ot_bytes"),
                            ("filter_transform", ST_KT, "kt_bytes")):
         ms, cnt = stage[idx]
         if cnt > 0:
-            b = sum(l.algorithmic()[key] * l.repeats for l in layers) * (cnt / launches_step)
+            who = staged if idx == ST_OT else layers
+            per_step = launches_step if idx == ST_OT else all_launches
+            b = sum(l.algorithmic()[key] * l.repeats for l in who) * (cnt / per_step)
             gbs = b / (ms * 1e-3) / 1e9
             transforms[name] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                 "frac": round(gbs / PEAK_HBM_GBS, 4), "launches": cnt}
 
+    if fused_stage[1] > 0:
+        fl = [l for l in layers if l.fused]
+        per_step = sum(l.repeats for l in fl)
+        fbytes = sum((256.0 * (l.K * l.C + l.C * l.plan.T) + 4.0 * l.N * l.K * l.H * l.H) * l.repeats for l in fl)
+        fflops = sum(l.algorithmic()["gemm_flops"] * l.repeats for l in fl)
+        k = fused_stage[1] / per_step
+        transforms["fused_gemm_output"] = {
+            "bound": "hbm", "achieved": round(fbytes * k / (fused_stage[0] * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
+            "unit": "GB/s", "frac": round(fbytes * k / (fused_stage[0] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+            "launches": fused_stage[1], "mfma_tflops": round(fflops * k / (fused_stage[0] * 1e-3) / 1e12, 2)}
+
     # per-layer detail, outside the timed region
     per_layer = []
-    L.timing(0x0f)
+    L.timing(0x4f)
     for lay in ([] if args.timed_only else layers):
         L.timing_reset()
         reps = 5
@@ -272,17 +303,21 @@ def main():
             forward(L, lay, V, M)
         L.sync()
         st = [L.stage_time(i)[0] / reps for i in range(4)]
+        if lay.fused:      # one kernel does the GEMM and the output transform: listed under gemm
+            st[ST_GEMM] = L.stage_time(6)[0] / reps
+            st[ST_OT] = 0.0
         total = sum(st)
         a = lay.algorithmic()
         g = L.wino_configs()[lay.plan.gemm_config]
         per_layer.append({
             "layer": "%d->%d@%d" % (lay.C, lay.K, lay.H), "batch": N, "repeats": lay.repeats,
+            "pipeline": "fused" if lay.fused else "staged",
             "tile": "%dx%dx%d" % (g.bm, g.bn, g.bk), "ms": round(total, 4),
             "gflops": round(lay.flops / (total * 1e-3) / 1e9, 1),
             "gemm_tflops": round(a["gemm_flops"] / (st[ST_GEMM] * 1e-3) / 1e12, 2),
             "gemm_frac_mfma": round(a["gemm_flops"] / (st[ST_GEMM] * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 3),
             "input_tran_gbs": round(a["it_bytes"] / (st[ST_IT] * 1e-3) / 1e9, 0),
-            "output_tran_gbs": round(a["ot_bytes"] / (st[ST_OT] * 1e-3) / 1e9, 0),
+            "output_tran_gbs": round(a["ot_bytes"] / (st[ST_OT] * 1e-3) / 1e9, 0) if st[ST_OT] else None,
             "stage_ms": {"kernel_tran": round(st[ST_KT], 4), "input_tran": round(st[ST_IT], 4),
                          "gemm": round(st[ST_GEMM], 4), "output_tran": round(st[ST_OT], 4)},
         })
@@ -293,7 +328,8 @@ def main():
         "value": round(value, 1), "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": args.workload, "description": desc, "batch": N, "algorithm": "winograd_f63_staged",
+        "config": {"workload": args.workload, "description": desc, "batch": N, "algorithm": "winograd_f63",
+                   "pipeline": args.pipeline + " (per layer: " + ",".join("fused" if l.fused else "staged" for l in layers) + ")",
                    "filter_transform": "offline" if filter_ready else "online (inside the timed region)",
                    "tuned": not args.no_tune, "stage_events": args.stage_events,
                    "device": info["arch"], "compute_units": info["compute_units"], "clock_mhz": info["clock_mhz"]},

@@ -88,6 +88,9 @@ _ABI = {
     "fc_wino_input_transform": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp]),
     "fc_wino_gemm": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, _vp]),
     "fc_wino_output_transform": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, C.c_int, _vp]),
+    "fc_wino_gemm_output_fused": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, _vp, C.c_int, _vp]),
+    "fc_wino_prefer_fused": (C.c_int, [C.POINTER(ConvShape)]),
+    "fc_wino_forward_fused": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, _vp, C.c_int, C.c_int, _vp, _vp, _vp]),
     "fc_wino_forward": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, _vp, C.c_int, C.c_int,
                                   _vp, _vp, _vp, _vp]),
     "fc_igemm_num_configs": (C.c_int, []),
@@ -266,6 +269,16 @@ class Library:
     def wino_output_transform(self, plan, M, y, bias=None, relu=False):
         self._check(self.c.fc_wino_output_transform(self.ctx, C.byref(plan), M, bias, int(relu), y))
 
+    def wino_gemm_output_fused(self, plan, U, V, y, bias=None, relu=False):
+        self._check(self.c.fc_wino_gemm_output_fused(self.ctx, C.byref(plan), U, V, bias, int(relu), y))
+
+    def wino_prefer_fused(self, shape):
+        return bool(self.c.fc_wino_prefer_fused(C.byref(shape)))
+
+    def wino_forward_fused(self, plan, x, w, U, V, y, bias=None, relu=False, filter_ready=False):
+        self._check(self.c.fc_wino_forward_fused(self.ctx, C.byref(plan), x, w, bias, int(relu),
+                                                 int(filter_ready), U, V, y))
+
     def wino_forward(self, plan, x, w, U, V, M, y, bias=None, relu=False, filter_ready=False):
         self._check(self.c.fc_wino_forward(self.ctx, C.byref(plan), x, w, bias, int(relu),
                                            int(filter_ready), U, V, M, y))
@@ -278,6 +291,22 @@ class Library:
         self._check(self.c.fc_conv_implicit_gemm(self.ctx, C.byref(plan), x, Wp, table, bias, int(relu), ws, y))
 
     # ---- whole-layer helpers over host arrays (tests, smoke)
+    def winograd_conv_fused(self, shape, x, w, bias=None, relu=False, config=None):
+        """Filter transform, input transform, then GEMM + output transform in one kernel."""
+        plan = self.wino_plan(shape, self.wino_default_config(shape) if config is None else config)
+        mark = self.mark()
+        try:
+            dx, dw = self.upload(x), self.upload(w)
+            db = self.upload(bias) if bias is not None else None
+            U, V = self.alloc(plan.U_bytes), self.alloc(plan.V_bytes)
+            y = self.alloc(4 * shape.N * shape.K * plan.OH * plan.OW)
+            self.wino_filter_transform(plan, dw, U)
+            self.wino_input_transform(plan, dx, V)
+            self.wino_gemm_output_fused(plan, U, V, y, db, relu)
+            return self.download(y, (shape.N, shape.K, plan.OH, plan.OW))
+        finally:
+            self.release(mark)
+
     def winograd_conv(self, shape, x, w, bias=None, relu=False, config=None, stages=False):
         plan = self.wino_plan(shape, self.wino_default_config(shape) if config is None else config)
         mark = C.c_size_t()

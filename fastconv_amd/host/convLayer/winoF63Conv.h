@@ -1,11 +1,12 @@
-// Winograd F(6x6,3x3) layer, blocked pipeline: the batch is cut into blocks of
-// `tileBlock` tiles (whole images) and the input transform, GEMM and output
-// transform run block after block over block-local V and M scratch, so the
-// 64-plane intermediates of one block stay in the 256 MB memory-side cache
-// instead of making a round trip through HBM.  The filter transform is always
-// done once in Init().  Interface of the reference's ConvWinoF63Layer
+// Winograd F(6x6,3x3) layer, blocked pipeline: the GEMM result of one block of
+// (32 output channels x 32 tiles x 64 frequencies) is consumed by the output
+// transform straight out of registers and LDS -- there is no whole-layer M
+// buffer -- and the batch may be cut into blocks of `tileBlock` tiles (whole
+// images) so that only one block of V exists at a time.  The filter transform is
+// always done once in Init().  Interface of the reference's ConvWinoF63Layer
 // (convLayer/winoF63Conv.h:4-209), whose scratch is likewise sized for one
-// (ocBlock x tileBlock) block (:161-166).
+// (ocBlock x tileBlock) block and whose GEMM output goes to the output
+// transform through a small buffer (winoF63/winoF63.cpp:1574-1737).
 #ifndef WINOF63CONV_H_
 #define WINOF63CONV_H_
 
@@ -50,7 +51,7 @@ class ConvWinoF63Layer : public ConvLayer {
     int imgBlock;
 
     float *inputBuf;    // V of one block, device
-    float *gemmBuf;     // M of one block, device
+    float *gemmBuf;     // unused: the products never leave the compute unit
     float *kernelBuf;   // U of the whole layer, device
 
     int gemmConfig_best;

@@ -183,6 +183,28 @@ int fc_wino_output_transform(fc_context *ctx, const fc_wino_plan *plan,
                              const float *M_dev, const float *bias_dev, int relu,
                              float *y_dev);
 
+/* GEMM and output transform in one kernel: the 64 per-frequency products of a
+ * block of (32 output channels x 32 tiles) stay in registers and LDS, M is never
+ * written (M_dev is not needed).  The counterpart of the reference's blocked
+ * pipeline, where the GEMM result of one block is consumed by the output
+ * transform out of block-local scratch (winoF63/winoF63.cpp:1574-1737).  Pays
+ * when the transformed filter fits in L2 (C*K up to about 8192); any plan whose
+ * C_pad is a multiple of 8 is accepted. */
+int fc_wino_gemm_output_fused(fc_context *ctx, const fc_wino_plan *plan,
+                              const float *U_dev, const float *V_dev,
+                              const float *bias_dev, int relu, float *y_dev);
+
+/* 1 when the fused kernel is expected to beat fc_wino_gemm + fc_wino_output_transform
+ * for this layer (measured on MI355X: when the transformed filter, 256*C*K bytes,
+ * stays L2-resident, C*K <= 8192), else 0. */
+int fc_wino_prefer_fused(const fc_conv_shape *shape);
+
+/* Filter transform (unless filter_ready), input transform, fused GEMM + output
+ * transform: the whole layer without an M buffer. */
+int fc_wino_forward_fused(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev,
+                          const float *w_dev, const float *bias_dev, int relu, int filter_ready,
+                          float *U_dev, float *V_dev, float *y_dev);
+
 /* All stages back to back: what winoF63_v1_single (winoF63ZC/winoF63ZC.h:5-6)
  * does in one call.  filter_ready != 0 skips the filter transform (U already
  * holds it: the "offline" strategy, ConvTest.cpp:230-243). */

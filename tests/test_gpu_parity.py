@@ -114,6 +114,35 @@ def test_winograd_bias_relu_epilogue(lib):
     assert O.max_rel_err(y, truth) <= TOL_WINO
 
 
+@pytest.mark.parametrize("shp", [
+    (2, 3, 8, 11, 5), (1, 64, 56, 56, 64), (3, 10, 14, 14, 70), (2, 16, 7, 7, 33), (1, 8, 30, 20, 40),
+    (1, 3, 224, 224, 64), (4, 64, 28, 28, 128), (2, 130, 13, 13, 40),
+])
+def test_winograd_fused_gemm_output_against_oracle(lib, shp):
+    """GEMM + output transform in one kernel (no M buffer): same tolerance as the staged
+    pipeline, and the same bits as the staged pipeline (same summation order)."""
+    s = O.shape(*shp)
+    x, w = O.make_inputs(s, seed=shp[1] + 17)
+    bias = O.rng_uniform(3, (s.K,))
+    announce("fused winograd", shp)
+    y = lib.winograd_conv_fused(cshape(s), x, w, bias=bias, relu=True)
+    truth = np.maximum(O.naive_conv_f64(s, x, w, bias), 0.0)
+    assert O.max_rel_err(y, truth) <= TOL_WINO
+    assert np.array_equal(y, lib.winograd_conv(cshape(s), x, w, bias=bias, relu=True))
+
+
+def test_winograd_fused_full_size_layers(lib):
+    for (N, C, H, K) in [(32, 3, 224, 64), (32, 64, 112, 128)]:
+        s = O.shape(N, C, H, H, K)
+        x, w = O.make_inputs(s, seed=2)
+        announce("fused full size", (N, C, H, K))
+        yf = lib.winograd_conv_fused(cshape(s), x, w)
+        yi = lib.implicit_gemm_conv(cshape(s), x, w)
+        assert O.max_rel_err(yf, yi) <= TOL_WINO
+        sub = O.shape(1, C, H, H, K)
+        assert O.max_rel_err(yf[:1], O.naive_conv_f64(sub, np.ascontiguousarray(x[:1]), w)) <= TOL_WINO
+
+
 def test_winograd_rejects_unsupported(lib):
     import fastconv_amd as F
     for bad in [O.shape(1, 4, 8, 8, 4, 3, 3, 2, 2, 1), O.shape(1, 4, 8, 8, 4, 5, 5, 1, 1, 2),
