@@ -29,21 +29,40 @@ PEAK_HBM_GBS = 8000.0
 # The counters need their own rocprofv3 runs, so this is not re-measured by every bench run.
 MEASURED_GEMM_TRAFFIC = {"vgg16_b32": 485.7e6}
 
-# (C, K, H, repeats)
+# (C, K, H, repeats): 3x3, stride 1, pad 1
 VGG16 = [(3, 64, 224, 1), (64, 64, 224, 1), (64, 128, 112, 1), (128, 128, 112, 1), (128, 256, 56, 1),
          (256, 256, 56, 2), (256, 512, 28, 1), (512, 512, 28, 2), (512, 512, 14, 3)]
 RESNET50_3X3 = [(64, 64, 56, 3), (128, 128, 28, 4), (256, 256, 14, 6), (512, 512, 7, 3)]
 STRESS = [(256, 256, 56, 1), (512, 512, 28, 1), (512, 512, 14, 1)]
+# (C, K, H, kernel, stride, pad, repeats): the ResNet-50 bottleneck layers of BASELINE config 4
+RESNET50 = [(3, 64, 224, 7, 2, 3, 1),
+            (64, 64, 56, 1, 1, 0, 1), (64, 64, 56, 3, 1, 1, 3), (64, 256, 56, 1, 1, 0, 4), (256, 64, 56, 1, 1, 0, 2),
+            (256, 128, 56, 1, 1, 0, 1), (128, 128, 56, 3, 2, 1, 1), (128, 128, 28, 3, 1, 1, 3),
+            (128, 512, 28, 1, 1, 0, 4), (512, 128, 28, 1, 1, 0, 3), (256, 512, 56, 1, 2, 0, 1),
+            (512, 256, 28, 1, 1, 0, 1), (256, 256, 28, 3, 2, 1, 1), (256, 256, 14, 3, 1, 1, 5),
+            (256, 1024, 14, 1, 1, 0, 6), (1024, 256, 14, 1, 1, 0, 5), (512, 1024, 28, 1, 2, 0, 1),
+            (1024, 512, 14, 1, 1, 0, 1), (512, 512, 14, 3, 2, 1, 1), (512, 512, 7, 3, 1, 1, 2),
+            (512, 2048, 7, 1, 1, 0, 3), (2048, 512, 7, 1, 1, 0, 2), (1024, 2048, 14, 1, 2, 0, 1)]
+IM2COL_ABC = [(256, 256, 56, 3, 1, 1, 1), (128, 256, 56, 3, 2, 1, 1), (256, 1024, 14, 1, 1, 0, 1)]
+
+
+def _w(layers):
+    return [(c, k, h, 3, 1, 1, r) for (c, k, h, r) in layers]
+
 
 WORKLOADS = {
-    # name: (layers, batch, description)
-    "vgg16_b32": (VGG16, 32, "VGG-16 conv stack, 13 layers, 3x3 s1 p1, Winograd F(6,3), batch 32"),
-    "vgg16_b1": (VGG16, 1, "VGG-16 conv stack, 13 layers, 3x3 s1 p1, Winograd F(6,3), batch 1"),
-    "resnet50_3x3_b32": (RESNET50_3X3, 32, "ResNet-50 3x3 s1 bottleneck convs, Winograd F(6,3), batch 32"),
-    "resnet50_3x3_b1": (RESNET50_3X3, 1, "ResNet-50 3x3 s1 bottleneck convs, Winograd F(6,3), batch 1"),
-    "cfg1": ([(64, 64, 56, 1)], 1, "single 3x3 conv 64->64 @56, batch 1"),
-    "stress_b64": (STRESS, 64, "VGG-16 256@56, 512@28, 512@14, batch 64"),
-    "stress_b128": (STRESS, 128, "VGG-16 256@56, 512@28, 512@14, batch 128"),
+    # name: (layers, batch, algorithm, description)
+    "vgg16_b32": (_w(VGG16), 32, "winograd", "VGG-16 conv stack, 13 layers, 3x3 s1 p1, Winograd F(6,3), batch 32"),
+    "vgg16_b1": (_w(VGG16), 1, "winograd", "VGG-16 conv stack, 13 layers, 3x3 s1 p1, Winograd F(6,3), batch 1"),
+    "vgg16_auto_b32": (_w(VGG16), 32, "auto", "VGG-16 conv stack, faster of Winograd / implicit GEMM per layer, batch 32"),
+    "resnet50_b32": (RESNET50, 32, "auto", "ResNet-50 conv layers (53 convs), auto algorithm per layer, batch 32"),
+    "resnet50_b1": (RESNET50, 1, "auto", "ResNet-50 conv layers (53 convs), auto algorithm per layer, batch 1"),
+    "resnet50_3x3_b32": (_w(RESNET50_3X3), 32, "winograd", "ResNet-50 3x3 s1 convs, Winograd F(6,3), batch 32"),
+    "resnet50_3x3_b1": (_w(RESNET50_3X3), 1, "winograd", "ResNet-50 3x3 s1 convs, Winograd F(6,3), batch 1"),
+    "im2col_abc_b1": (IM2COL_ABC, 1, "im2col", "BASELINE config 2: 3x3 256@56, 3x3 s2 128->256@56, 1x1 256->1024@14, batch 1"),
+    "cfg1": (_w([(64, 64, 56, 1)]), 1, "winograd", "single 3x3 conv 64->64 @56, batch 1"),
+    "stress_b64": (_w(STRESS), 64, "winograd", "VGG-16 256@56, 512@28, 512@14, batch 64"),
+    "stress_b128": (_w(STRESS), 128, "winograd", "VGG-16 256@56, 512@28, 512@14, batch 128"),
 }
 
 ST_KT, ST_IT, ST_GEMM, ST_OT = 0, 1, 2, 3
@@ -56,17 +75,26 @@ def log(*a):
 class Layer:
     """One conv layer with its buffers resident on the device."""
 
-    def __init__(self, L, F, N, C, K, H, repeats, rng):
-        self.N, self.C, self.K, self.H, self.repeats = N, C, K, H, repeats
-        self.shape = F.ConvShape(N, C, H, H, K, 3, 3, 1, 1, 1, 1, 1, 1)
+    def __init__(self, L, F, N, spec, rng):
+        C, K, H, ks, st, pad, repeats = spec
+        self.N, self.C, self.K, self.H, self.ks, self.st, self.pad, self.repeats = N, C, K, H, ks, st, pad, repeats
+        self.shape = F.ConvShape(N, C, H, H, K, ks, ks, st, st, pad, pad, pad, pad)
+        self.OH = self.shape.out_hw()[0]
         x = rng.random((N, C, H, H), dtype=np.float32) * 2.0 - 1.0
-        w = (rng.standard_normal((K, C, 3, 3), dtype=np.float32) * np.float32(np.sqrt(2.0 / (9 * C))))
+        w = (rng.standard_normal((K, C, ks, ks), dtype=np.float32) * np.float32(np.sqrt(2.0 / (ks * ks * C))))
         self.x, self.w = L.upload(x), L.upload(w)
-        self.y = L.alloc(4 * N * K * H * H)
+        self.y = L.alloc(4 * N * K * self.OH * self.OH)
         self.flops = self.shape.flops()
-        self.plan = None
+        self.algo = "winograd"        # or "im2col"
+        self.plan = None              # Winograd plan
         self.U = None
         self.fused = False
+        self.iplan = self.Wp = self.table = self.ws = None   # implicit GEMM
+        self.wino_ok = ks == 3 and st == 1
+
+    def name(self):
+        tag = "" if (self.ks, self.st) == (3, 1) else " %dx%d/s%d" % (self.ks, self.ks, self.st)
+        return "%d->%d@%d%s" % (self.C, self.K, self.H, tag)
 
     def algorithmic(self):
         """Per-launch algorithmic work of each stage (flops for the GEMM, bytes for the transforms)."""
@@ -78,18 +106,38 @@ class Layer:
             "ot_bytes": 256.0 * self.K * T + 4.0 * self.N * self.K * self.H * self.H,
         }
 
+    def setup_im2col(self, L, cfg):
+        self.iplan = L.igemm_plan(self.shape, cfg)
+        self.Wp, self.table = L.alloc(self.iplan.Wp_bytes), L.alloc(self.iplan.table_bytes)
+        self.ws = L.alloc(self.iplan.ws_bytes) if self.iplan.ws_bytes else None
+        L.igemm_pack_filter(self.iplan, self.w, self.Wp, self.table)
+
 
 def forward(L, lay, V, M, filter_ready=False):
-    """One layer pass: staged (four kernels) or fused (GEMM + output transform in one kernel)."""
-    if lay.fused:
+    """One layer pass: implicit GEMM, or Winograd staged (four kernels) or fused (GEMM + output
+    transform in one kernel)."""
+    if lay.algo == "im2col":
+        L.conv_implicit_gemm(lay.iplan, lay.x, lay.Wp, lay.table, lay.y, ws=lay.ws)
+    elif lay.fused:
         L.wino_forward_fused(lay.plan, lay.x, lay.w, lay.U, V, lay.y, filter_ready=filter_ready)
     else:
         L.wino_forward(lay.plan, lay.x, lay.w, lay.U, V, M, lay.y, filter_ready=filter_ready)
 
 
+def _time(L, fn, iters):
+    fn()
+    L.sync()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        fn()
+    L.sync()
+    return (time.perf_counter() - t0) / iters * 1e3
+
+
 def tune_layer(L, lay, V, M, scratch_bytes, iters=3):
-    """Pick the GEMM tile shape with the shortest whole-layer forward."""
+    """Pick the GEMM tile shape and pipeline with the shortest whole-layer forward."""
     best = (None, False, 1e30)
+    lay.algo = "winograd"
     for cfg in L.wino_configs():
         plan = L.wino_plan(lay.shape, cfg.id)
         if plan.V_bytes > scratch_bytes[0] or plan.M_bytes > scratch_bytes[1]:
@@ -102,16 +150,23 @@ def tune_layer(L, lay, V, M, scratch_bytes, iters=3):
         # the fused kernel has one tile shape of its own; the plan only fixes the padding it reads
         for fused in ((False, True) if lay.C * lay.K <= 16384 else (False,)):
             lay.fused = fused
-            forward(L, lay, V, M)
-            L.sync()
-            t0 = time.perf_counter()
-            for _ in range(iters):
-                forward(L, lay, V, M)
-            L.sync()
-            ms = (time.perf_counter() - t0) / iters * 1e3
+            ms = _time(L, lambda: forward(L, lay, V, M), iters)
             if ms < best[2]:
                 best = (cfg.id, fused, ms)
         L.release(mark)
+    return best
+
+
+def tune_im2col(L, lay, iters=3):
+    best = (None, 1e30)
+    lay.algo = "im2col"
+    for cfg in L.igemm_configs():
+        mark = L.mark()
+        lay.setup_im2col(L, cfg.id)
+        ms = _time(L, lambda: forward(L, lay, None, None), iters)
+        L.release(mark)
+        if ms < best[1]:
+            best = (cfg.id, ms)
     return best
 
 
@@ -193,37 +248,70 @@ def main():
         sys.exit(2)
 
     import fastconv_amd as F
-    layers_def, N, desc = WORKLOADS[args.workload]
+    layers_def, N, algo, desc = WORKLOADS[args.workload]
     rng = np.random.default_rng(0)
 
-    # arena: activations + filters + U per layer, one shared V and M (largest layer)
-    act = sum(4 * N * (C + K) * H * H for (C, K, H, _) in layers_def)
+    # arena: activations + filters + U / packed filter per layer, one shared V and M (largest layer)
+    act = sum(4 * N * (C * H * H + K * (H // st + 1) ** 2) for (C, K, H, ks, st, pad, _) in layers_def)
     tiles = lambda H: N * ((H + 5) // 6) ** 2
-    vmax = max(256 * (C + 32) * (tiles(H) + 256) for (C, K, H, _) in layers_def)
-    mmax = max(256 * max(2 * K if K < 128 else K + 128, 128) * (tiles(H) + 256) for (C, K, H, _) in layers_def)
-    umax = sum(256 * (C + 32) * (K + 256) for (C, K, H, _) in layers_def) * 2
-    pool = int(act + vmax + mmax + umax + (512 << 20))
+    wl = [(C, K, H) for (C, K, H, ks, st, pad, _) in layers_def if ks == 3 and st == 1 and algo != "im2col"]
+    vmax = max([256 * (C + 32) * (tiles(H) + 256) for (C, K, H) in wl] + [256])
+    mmax = max([256 * max(2 * K if K < 128 else K + 128, 128) * (tiles(H) + 256) for (C, K, H) in wl] + [256])
+    umax = sum(256 * (C + 32) * (K + 256) for (C, K, H) in wl) * 2
+    imax = sum(4 * (C * ks * ks + 32) * (K + 256) * 2 + 32 * 4 * N * K * (H // st + 1) ** 2 * (1 if N == 1 else 0)
+               for (C, K, H, ks, st, pad, _) in layers_def) + (256 << 20)
+    pool = int(act + vmax + mmax + umax + imax + (512 << 20))
     L = F.load(0, pool)
     info = L.device_info()
     log("device:", info)
     V, M = L.alloc(vmax), L.alloc(mmax)
-    layers = [Layer(L, F, N, C, K, H, rep, rng) for (C, K, H, rep) in layers_def]
+    layers = [Layer(L, F, N, spec, rng) for spec in layers_def]
 
     # tile shape per layer
     for lay in layers:
-        if args.no_tune:      # the library's untuned choices
-            cfg, fused, ms = L.wino_default_config(lay.shape), L.wino_prefer_fused(lay.shape), 0.0
+        want_wino = lay.wino_ok and algo in ("winograd", "auto")
+        want_im2col = algo == "im2col" or not lay.wino_ok or algo == "auto"
+        if algo == "winograd" and not lay.wino_ok:
+            raise SystemExit("workload %s: Winograd needs 3x3 stride 1" % args.workload)
+        wres = ires = None
+        if want_wino:
+            if args.no_tune:      # the library's untuned choices
+                wres = (L.wino_default_config(lay.shape), L.wino_prefer_fused(lay.shape), 0.0)
+            else:
+                wres = tune_layer(L, lay, V, M, (vmax, mmax))
+        if want_im2col:
+            if args.no_tune:
+                ires = (L.igemm_default_config(lay.shape), 0.0)
+            else:
+                ires = tune_im2col(L, lay)
+        if wres and ires:
+            if args.no_tune:      # the driver's rule for -a auto: Winograd unless few channels or few tiles
+                T = N * ((lay.H + 5) // 6) ** 2
+                use_w = not (lay.C < 16 or (T < 64 and lay.C * lay.K >= 128 * 128))
+            else:
+                use_w = wres[2] <= ires[1]
         else:
-            cfg, fused, ms = tune_layer(L, lay, V, M, (vmax, mmax))
-        if args.pipeline != "auto":
-            fused = args.pipeline == "fused"
-        lay.fused = fused
-        lay.plan = L.wino_plan(lay.shape, cfg)
-        lay.U = L.alloc(lay.plan.U_bytes)
-        L.wino_filter_transform(lay.plan, lay.w, lay.U)
-        g = L.wino_configs()[cfg]
-        log("layer %d->%d @%d: %s, tile %dx%dx%d (cfg %d) %.3f ms"
-            % (lay.C, lay.K, lay.H, "fused" if fused else "staged", g.bm, g.bn, g.bk, cfg, ms))
+            use_w = wres is not None
+        if use_w:
+            cfg, fused, ms = wres
+            if args.pipeline != "auto":
+                fused = args.pipeline == "fused"
+            lay.algo, lay.fused = "winograd", fused
+            lay.plan = L.wino_plan(lay.shape, cfg)
+            lay.U = L.alloc(lay.plan.U_bytes)
+            L.wino_filter_transform(lay.plan, lay.w, lay.U)
+            g = L.wino_configs()[cfg]
+            log("layer %s: winograd %s, tile %dx%dx%d (cfg %d) %.3f ms%s"
+                % (lay.name(), "fused" if fused else "staged", g.bm, g.bn, g.bk, cfg, ms,
+                   " (im2col %.3f ms)" % ires[1] if ires else ""))
+        else:
+            cfg, ms = ires
+            lay.algo = "im2col"
+            lay.setup_im2col(L, cfg)
+            g = L.igemm_configs()[cfg]
+            log("layer %s: im2col, tile %dx%dx%d (cfg %d) split %d %.3f ms%s"
+                % (lay.name(), g.bm, g.bn, g.bk, cfg, lay.iplan.split_k, ms,
+                   " (winograd %.3f ms)" % wres[2] if wres else ""))
     L.sync()
 
     filter_ready = args.offline_filter
@@ -237,7 +325,7 @@ def main():
         step()
     L.sync()
 
-    mask = {"all": 0x4f, "gemm": 1 << ST_GEMM, "none": 0}[args.stage_events]
+    mask = {"all": 0x5f, "gemm": (1 << ST_GEMM) | (1 << 4), "none": 0}[args.stage_events]
     L.timing(mask)
     L.timing_reset()
     t0 = time.perf_counter()
@@ -247,6 +335,7 @@ def main():
     elapsed = time.perf_counter() - t0
     stage = [L.stage_time(i) for i in range(4)]
     fused_stage = L.stage_time(6)
+    igemm_stage = L.stage_time(4)
     L.timing(0)
 
     ms_per_step = elapsed / args.steps * 1e3
@@ -254,7 +343,8 @@ def main():
     value = step_flops / (ms_per_step * 1e-3) / 1e9
 
     # dominant kernel: the batched GEMM. achieved = algorithmic flops of all its launches / their event time
-    staged = [l for l in layers if not l.fused]
+    wino = [l for l in layers if l.algo == "winograd"]
+    staged = [l for l in wino if not l.fused]
     gemm_flops_step = sum(l.algorithmic()["gemm_flops"] * l.repeats for l in staged)
     launches_step = max(1, sum(l.repeats for l in staged))
     roofline = {"kernel": "wino_gemm_kernel", "bound": "mfma", "achieved": None, "peak": PEAK_MFMA_F32_TFLOPS,
@@ -269,12 +359,12 @@ def main():
                         launches=gemm_cnt, avg_launch_ms=round(gemm_ms / gemm_cnt, 5),
                         flops_per_launch_avg=gemm_flops_step / launches_step)
     transforms = {}
-    all_launches = sum(l.repeats for l in layers)
+    all_launches = max(1, sum(l.repeats for l in wino))
     for name, idx, key in (("input_transform", ST_IT, "it_bytes"), ("output_transform", ST_OT, "ot_bytes"),
                            ("filter_transform", ST_KT, "kt_bytes")):
         ms, cnt = stage[idx]
         if cnt > 0:
-            who = staged if idx == ST_OT else layers
+            who = staged if idx == ST_OT else wino
             per_step = launches_step if idx == ST_OT else all_launches
             b = sum(l.algorithmic()[key] * l.repeats for l in who) * (cnt / per_step)
             gbs = b / (ms * 1e-3) / 1e9
@@ -282,7 +372,7 @@ def main():
                                 "frac": round(gbs / PEAK_HBM_GBS, 4), "launches": cnt}
 
     if fused_stage[1] > 0:
-        fl = [l for l in layers if l.fused]
+        fl = [l for l in wino if l.fused]
         per_step = sum(l.repeats for l in fl)
         fbytes = sum((256.0 * (l.K * l.C + l.C * l.plan.T) + 4.0 * l.N * l.K * l.H * l.H) * l.repeats for l in fl)
         fflops = sum(l.algorithmic()["gemm_flops"] * l.repeats for l in fl)
@@ -292,35 +382,52 @@ def main():
             "unit": "GB/s", "frac": round(fbytes * k / (fused_stage[0] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
             "launches": fused_stage[1], "mfma_tflops": round(fflops * k / (fused_stage[0] * 1e-3) / 1e12, 2)}
 
+    if igemm_stage[1] > 0:
+        il = [l for l in layers if l.algo == "im2col"]
+        per_step = sum(l.repeats for l in il)
+        iflops = sum(l.flops * l.repeats for l in il) * (igemm_stage[1] / per_step)
+        tf = iflops / (igemm_stage[0] * 1e-3) / 1e12
+        transforms["implicit_gemm"] = {"bound": "mfma", "achieved": round(tf, 2), "peak": PEAK_MFMA_F32_TFLOPS,
+                                       "unit": "TFLOP/s", "frac": round(tf / PEAK_MFMA_F32_TFLOPS, 4),
+                                       "launches": igemm_stage[1]}
+    if not staged and igemm_stage[1] > 0:      # no staged Winograd layer: the implicit GEMM is the dominant kernel
+        roofline = dict(transforms["implicit_gemm"], kernel="igemm_conv_kernel", traffic=None,
+                        avg_launch_ms=round(igemm_stage[0] / igemm_stage[1], 5))
+
     # per-layer detail, outside the timed region
     per_layer = []
-    L.timing(0x4f)
+    L.timing(0x5f)
     for lay in ([] if args.timed_only else layers):
         L.timing_reset()
         reps = 5
-        t0 = time.perf_counter()
         for _ in range(reps):
             forward(L, lay, V, M)
         L.sync()
-        st = [L.stage_time(i)[0] / reps for i in range(4)]
-        if lay.fused:      # one kernel does the GEMM and the output transform: listed under gemm
-            st[ST_GEMM] = L.stage_time(6)[0] / reps
-            st[ST_OT] = 0.0
-        total = sum(st)
-        a = lay.algorithmic()
-        g = L.wino_configs()[lay.plan.gemm_config]
-        per_layer.append({
-            "layer": "%d->%d@%d" % (lay.C, lay.K, lay.H), "batch": N, "repeats": lay.repeats,
-            "pipeline": "fused" if lay.fused else "staged",
-            "tile": "%dx%dx%d" % (g.bm, g.bn, g.bk), "ms": round(total, 4),
-            "gflops": round(lay.flops / (total * 1e-3) / 1e9, 1),
-            "gemm_tflops": round(a["gemm_flops"] / (st[ST_GEMM] * 1e-3) / 1e12, 2),
-            "gemm_frac_mfma": round(a["gemm_flops"] / (st[ST_GEMM] * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 3),
-            "input_tran_gbs": round(a["it_bytes"] / (st[ST_IT] * 1e-3) / 1e9, 0),
-            "output_tran_gbs": round(a["ot_bytes"] / (st[ST_OT] * 1e-3) / 1e9, 0) if st[ST_OT] else None,
-            "stage_ms": {"kernel_tran": round(st[ST_KT], 4), "input_tran": round(st[ST_IT], 4),
-                         "gemm": round(st[ST_GEMM], 4), "output_tran": round(st[ST_OT], 4)},
-        })
+        g = (L.igemm_configs()[lay.iplan.config] if lay.algo == "im2col" else L.wino_configs()[lay.plan.gemm_config])
+        row = {"layer": lay.name(), "batch": N, "repeats": lay.repeats, "algorithm": lay.algo,
+               "tile": "%dx%dx%d" % (g.bm, g.bn, g.bk)}
+        if lay.algo == "im2col":
+            ms = L.stage_time(4)[0] / reps
+            row.update(ms=round(ms, 4), gflops=round(lay.flops / (ms * 1e-3) / 1e9, 1), split_k=lay.iplan.split_k,
+                       gemm_tflops=round(lay.flops / (ms * 1e-3) / 1e12, 2),
+                       gemm_frac_mfma=round(lay.flops / (ms * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 3))
+        else:
+            st = [L.stage_time(i)[0] / reps for i in range(4)]
+            if lay.fused:      # one kernel does the GEMM and the output transform: listed under gemm
+                st[ST_GEMM] = L.stage_time(6)[0] / reps
+                st[ST_OT] = 0.0
+            total = sum(st)
+            a = lay.algorithmic()
+            row.update({
+                "pipeline": "fused" if lay.fused else "staged", "ms": round(total, 4),
+                "gflops": round(lay.flops / (total * 1e-3) / 1e9, 1),
+                "gemm_tflops": round(a["gemm_flops"] / (st[ST_GEMM] * 1e-3) / 1e12, 2),
+                "gemm_frac_mfma": round(a["gemm_flops"] / (st[ST_GEMM] * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 3),
+                "input_tran_gbs": round(a["it_bytes"] / (st[ST_IT] * 1e-3) / 1e9, 0),
+                "output_tran_gbs": round(a["ot_bytes"] / (st[ST_OT] * 1e-3) / 1e9, 0) if st[ST_OT] else None,
+                "stage_ms": {"kernel_tran": round(st[ST_KT], 4), "input_tran": round(st[ST_IT], 4),
+                             "gemm": round(st[ST_GEMM], 4), "output_tran": round(st[ST_OT], 4)}})
+        per_layer.append(row)
     L.timing(0)
 
     out = {
@@ -328,8 +435,9 @@ def main():
         "value": round(value, 1), "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": args.workload, "description": desc, "batch": N, "algorithm": "winograd_f63",
-                   "pipeline": args.pipeline + " (per layer: " + ",".join("fused" if l.fused else "staged" for l in layers) + ")",
+        "config": {"workload": args.workload, "description": desc, "batch": N, "algorithm": algo,
+                   "per_layer": ",".join("im2col" if l.algo == "im2col" else ("wino-fused" if l.fused else "wino-staged")
+                                         for l in layers),
                    "filter_transform": "offline" if filter_ready else "online (inside the timed region)",
                    "tuned": not args.no_tune, "stage_events": args.stage_events,
                    "device": info["arch"], "compute_units": info["compute_units"], "clock_mhz": info["clock_mhz"]},
