@@ -106,7 +106,21 @@ __device__ __forceinline__ void ig_scatter_rows(float *lds, const float (&r)[siz
     ((lds[I * rowStride] = r[I]), ...);
 }
 
-template <class TL>
+// Predicated 16-byte row copies for the pointwise (1x1, stride 1, no padding) case, where
+// the column matrix IS the input: row c of it is channel c of x, contiguous over the pixels.
+template <int... I>
+__device__ __forceinline__ void ig_load_rows_pw(floatx4 (&r)[sizeof...(I)], const float *p, size_t rowStride, int row0,
+                                                int rowStep, int rowLimit, bool valid,
+                                                std::integer_sequence<int, I...>) {
+    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+    ((r[I] = (valid && row0 + I * rowStep < rowLimit) ? *reinterpret_cast<const floatx4 *>(p + (size_t)I * rowStride)
+                                                       : zero),
+     ...);
+}
+
+// PW: pointwise layers whose pixels-per-image count is a multiple of 4 copy the B tile as
+// 16-byte vectors (four pixels of one channel) instead of gathering it element by element.
+template <class TL, bool PW>
 __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmParams p) {
     constexpr int BM = TL::BM_, BN = TL::BN_, BK = TL::BK_;
     constexpr int MI = TL::MI, NI = TL::NI, A_LD = TL::A_LD, B_LD = TL::B_LD;
@@ -144,6 +158,26 @@ __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmPara
     }
     const int bLds = grow0 * BN + gcol;
 
+    // pointwise: this thread's 4-pixel column group and first row of each copy pass
+    constexpr int BV_LD = BK * BN / 4 / TL::THREADS, BV_ROWS = TL::THREADS * 4 / BN;
+    static_assert((BK * BN / 4) % TL::THREADS == 0, "every thread copies the same number of float4");
+    using SeqBV = std::make_integer_sequence<int, BV_LD>;
+    const int vrow = tid / (BN / 4), vcol = (tid % (BN / 4)) * 4;
+    const int HW = p.H * p.W;
+    const float *vg = p.x;
+    bool vvalid = false;
+    if (PW) {
+        const long pix4 = (long)pb * BN + vcol;
+        vvalid = pix4 < p.Npix;
+        if (vvalid) {
+            const uint32_t n = fc_div((uint32_t)pix4, p.divOHW);
+            vg = p.x + ((size_t)n * p.C + vrow) * HW + ((uint32_t)pix4 - n * (uint32_t)HW);
+        }
+    }
+    const size_t vPass = (size_t)BV_ROWS * HW, vStage = (size_t)BK * HW;
+    const int vLds = vrow * BN + vcol;
+    floatx4 rv[BV_LD];
+
     using SeqA = std::make_integer_sequence<int, A_LD>;
     using SeqB = std::make_integer_sequence<int, B_LD>;
     floatx4 ra[A_LD];
@@ -153,7 +187,12 @@ __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmPara
     const int sBegin = blockIdx.y * p.stagesPerSplit, sEnd = min(sBegin + p.stagesPerSplit, nStagesAll);
     ag += (size_t)sBegin * aStage;
     ig_load_rows(ra, ag, aPass, SeqA());
-    ig_gather_rows(rb, ximg, pixOff, maskR, maskS, p.table, sBegin * BK + grow0, TL::ROW_STEP, SeqB());
+    if (PW) {
+        vg += (size_t)sBegin * vStage;
+        ig_load_rows_pw(rv, vg, vPass, sBegin * BK + vrow, BV_ROWS, p.C, vvalid, SeqBV());
+    } else {
+        ig_gather_rows(rb, ximg, pixOff, maskR, maskS, p.table, sBegin * BK + grow0, TL::ROW_STEP, SeqB());
+    }
 
     floatx16 acc[MI][NI];
 #pragma unroll
@@ -164,7 +203,8 @@ __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmPara
             for (int i = 0; i < 16; i++) acc[mi][ni][i] = 0.f;
 
     ig_store_rows(&As[0][aLds], ra, TL::A_ROWS * BM, SeqA());
-    ig_scatter_rows(&Bs[0][bLds], rb, TL::ROW_STEP * BN, SeqB());
+    if (PW) ig_store_rows(&Bs[0][vLds], rv, BV_ROWS * BN, SeqBV());
+    else ig_scatter_rows(&Bs[0][bLds], rb, TL::ROW_STEP * BN, SeqB());
     __syncthreads();
 
     const int lrow = lane >> 5, lcol = lane & 31;
@@ -176,7 +216,12 @@ __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmPara
         if (more) {
             ag += aStage;
             ig_load_rows(ra, ag, aPass, SeqA());
-            ig_gather_rows(rb, ximg, pixOff, maskR, maskS, p.table, (s + 1) * BK + grow0, TL::ROW_STEP, SeqB());
+            if (PW) {
+                vg += vStage;
+                ig_load_rows_pw(rv, vg, vPass, (s + 1) * BK + vrow, BV_ROWS, p.C, vvalid, SeqBV());
+            } else {
+                ig_gather_rows(rb, ximg, pixOff, maskR, maskS, p.table, (s + 1) * BK + grow0, TL::ROW_STEP, SeqB());
+            }
         }
         float a[2][MI], bb[2][NI];
 #pragma unroll
@@ -200,7 +245,8 @@ __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmPara
         }
         if (more) {
             ig_store_rows(&As[buf ^ 1][aLds], ra, TL::A_ROWS * BM, SeqA());
-            ig_scatter_rows(&Bs[buf ^ 1][bLds], rb, TL::ROW_STEP * BN, SeqB());
+            if (PW) ig_store_rows(&Bs[buf ^ 1][vLds], rv, BV_ROWS * BN, SeqBV());
+            else ig_scatter_rows(&Bs[buf ^ 1][bLds], rb, TL::ROW_STEP * BN, SeqB());
         }
         __syncthreads();
     }
@@ -284,7 +330,10 @@ const int kNumIgConfigs = sizeof(kIgConfigs) / sizeof(kIgConfigs[0]);
 template <class TL>
 void launch(fc_context *ctx, IgemmParams &p) {
     const dim3 grid((unsigned)(p.nKB * p.nPB), (unsigned)p.splitK);
-    igemm_conv_kernel<TL><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
+    const bool pointwise = p.kh == 1 && p.kw == 1 && p.sh == 1 && p.sw == 1 && p.pt == 0 && p.pl == 0 &&
+                           p.OH == p.H && p.OW == p.W && (p.H * p.W) % 4 == 0 && ((uintptr_t)p.x & 15) == 0;
+    if (pointwise) igemm_conv_kernel<TL, true><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
+    else igemm_conv_kernel<TL, false><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
 }
 
 }  // namespace

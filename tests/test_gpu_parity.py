@@ -161,6 +161,9 @@ IGEMM_SHAPES = [
     (1, 256, 56, 56, 128, 1, 1, 2, 2, 0),        # 1x1 stride-2 projection
     (2, 2048, 7, 7, 512, 1, 1, 1, 1, 0),
     (1, 1, 5, 5, 1, 3, 3, 1, 1, 1), (3, 5, 9, 8, 70, 3, 2, 2, 1, 1), (2, 7, 15, 15, 33, 5, 5, 3, 3, 2),
+    # pointwise layers: vector path (pixels per image a multiple of 4) and gather path (7x7 = 49 pixels)
+    (32, 64, 56, 56, 256, 1, 1, 1, 1, 0), (3, 70, 6, 6, 33, 1, 1, 1, 1, 0), (5, 20, 7, 7, 40, 1, 1, 1, 1, 0),
+    (2, 19, 10, 10, 130, 1, 1, 1, 1, 0),
 ]
 
 
