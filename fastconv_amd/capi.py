@@ -75,6 +75,7 @@ _ABI = {
     "fc_upload": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
     "fc_download": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
     "fc_fill_zero": (C.c_int, [_vp, _vp, C.c_size_t]),
+    "fc_maxpool2x2": (C.c_int, [_vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int]),
     "fc_device_copy": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
     "fc_timing_enable": (C.c_int, [_vp, C.c_int]),
     "fc_timing_reset": (C.c_int, [_vp]),
@@ -193,6 +194,9 @@ class Library:
 
     def device_copy(self, dst, src, nbytes):
         self._check(self.c.fc_device_copy(self.ctx, dst, src, nbytes))
+
+    def maxpool2x2(self, x, y, N, Cc, H, W):
+        self._check(self.c.fc_maxpool2x2(self.ctx, x, y, N, Cc, H, W))
 
     def sync(self):
         self._check(self.c.fc_sync(self.ctx))

@@ -242,6 +242,30 @@ extern "C" int fc_device_copy(fc_context *ctx, void *dst_dev, const void *src_de
     return FC_OK;
 }
 
+__global__ __launch_bounds__(256) void fc_maxpool2x2_kernel(const float *__restrict__ x, float *__restrict__ y, long planes,
+                                                            int H, int W, int OH, int OW) {
+    const long total = planes * OH * OW;
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+        const long pl = i / ((long)OH * OW);
+        const int r = (int)(i - pl * OH * OW), oh = r / OW, ow = r - oh * OW;
+        const float *src = x + (pl * H + 2 * oh) * W + 2 * ow;
+        y[i] = fmaxf(fmaxf(src[0], src[1]), fmaxf(src[W], src[W + 1]));
+    }
+}
+
+extern "C" int fc_maxpool2x2(fc_context *ctx, const float *x_dev, float *y_dev, int N, int C, int H, int W) {
+    if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    if (!x_dev || !y_dev || N <= 0 || C <= 0 || H < 2 || W < 2)
+        return fc_set_error(ctx, FC_ERR_INVALID, "fc_maxpool2x2: bad argument", hipSuccess);
+    const int OH = H / 2, OW = W / 2;
+    const long total = (long)N * C * OH * OW;
+    long blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    fc_maxpool2x2_kernel<<<dim3((unsigned)blocks), dim3(256), 0, ctx->stream>>>(x_dev, y_dev, (long)N * C, H, W, OH, OW);
+    FC_LAUNCH_CHECK(ctx, "fc_maxpool2x2_kernel");
+    return FC_OK;
+}
+
 // --------------------------------------------------------------- timing
 
 static int fc_timing_fold(fc_context *ctx) {

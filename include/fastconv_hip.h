@@ -251,6 +251,14 @@ int fc_conv_implicit_gemm(fc_context *ctx, const fc_igemm_plan *plan, const floa
                           const float *Wp_dev, const int32_t *table_dev,
                           const float *bias_dev, int relu, float *ws_dev, float *y_dev);
 
+/* ---- glue for running layers back to back ---------------------------- */
+
+/* 2x2 max pooling, stride 2, NCHW, floor((H)/2) x floor((W)/2) output: the step between
+ * the convolution blocks of a VGG-style stack.  No counterpart in the reference (it has
+ * no layer but convolution); it exists so that a whole conv trunk can run on the device
+ * without host round trips (the layer graph of layer.h:29-84). */
+int fc_maxpool2x2(fc_context *ctx, const float *x_dev, float *y_dev, int N, int C, int H, int W);
+
 #ifdef __cplusplus
 }
 #endif
