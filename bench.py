@@ -88,9 +88,20 @@ class Layer:
         self.algo = "winograd"        # or "im2col"
         self.plan = None              # Winograd plan
         self.U = None
-        self.fused = False
+        self.pipe = "staged"          # Winograd pipeline: staged, fused (GEMM + output transform) or onepass
+        self.oplan = self.U2 = None   # single-kernel path: its plan and its filter layout
         self.iplan = self.Wp = self.table = self.ws = None   # implicit GEMM
         self.wino_ok = ks == 3 and st == 1
+
+    @property
+    def fused(self):
+        return self.pipe == "fused"
+
+    def setup_onepass(self, L):
+        if self.oplan is None:
+            self.oplan = L.wino_onepass_plan(self.shape)
+            self.U2 = L.alloc(self.oplan.U_bytes)
+            L.wino_onepass_filter_transform(self.oplan, self.w, self.U2)
 
     def name(self):
         tag = "" if (self.ks, self.st) == (3, 1) else " %dx%d/s%d" % (self.ks, self.ks, self.st)
@@ -118,6 +129,8 @@ def forward(L, lay, V, M, filter_ready=False):
     transform in one kernel)."""
     if lay.algo == "im2col":
         L.conv_implicit_gemm(lay.iplan, lay.x, lay.Wp, lay.table, lay.y, ws=lay.ws)
+    elif lay.pipe == "onepass":
+        L.wino_forward_onepass(lay.oplan, lay.x, lay.w, lay.U2, lay.y, filter_ready=filter_ready)
     elif lay.fused:
         L.wino_forward_fused(lay.plan, lay.x, lay.w, lay.U, V, lay.y, filter_ready=filter_ready)
     else:
@@ -136,7 +149,7 @@ def _time(L, fn, iters):
 
 def tune_layer(L, lay, V, M, scratch_bytes, iters=3):
     """Pick the GEMM tile shape and pipeline with the shortest whole-layer forward."""
-    best = (None, False, 1e30)
+    best = (None, "staged", 1e30)
     lay.algo = "winograd"
     for cfg in L.wino_configs():
         plan = L.wino_plan(lay.shape, cfg.id)
@@ -148,12 +161,18 @@ def tune_layer(L, lay, V, M, scratch_bytes, iters=3):
         mark = L.mark()
         lay.U = L.alloc(plan.U_bytes)
         # the fused kernel has one tile shape of its own; the plan only fixes the padding it reads
-        for fused in ((False, True) if lay.C * lay.K <= 16384 else (False,)):
-            lay.fused = fused
+        for pipe in (("staged", "fused") if lay.C * lay.K <= 16384 else ("staged",)):
+            lay.pipe = pipe
             ms = _time(L, lambda: forward(L, lay, V, M), iters)
             if ms < best[2]:
-                best = (cfg.id, fused, ms)
+                best = (cfg.id, pipe, ms)
         L.release(mark)
+    if lay.C <= 128:      # the whole layer in one kernel: no tile shape to choose
+        lay.setup_onepass(L)
+        lay.pipe = "onepass"
+        ms = _time(L, lambda: forward(L, lay, V, M), iters)
+        if ms < best[2]:
+            best = (best[0], "onepass", ms)
     return best
 
 
@@ -233,7 +252,7 @@ def main():
                     help="which kernels are bracketed by events inside the timed region (default: the dominant "
                          "kernel only; an event pair costs about 5 us per launch, so the other kernels are "
                          "bracketed in a few extra untimed steps after it)")
-    ap.add_argument("--pipeline", default="auto", choices=["auto", "staged", "fused"],
+    ap.add_argument("--pipeline", default="auto", choices=["auto", "staged", "fused", "onepass"],
                     help="Winograd pipeline per layer: four staged kernels, GEMM + output transform fused, or "
                          "whichever is faster for the layer (auto)")
     ap.add_argument("--timed-only", action="store_true",
@@ -278,7 +297,9 @@ def main():
         wres = ires = None
         if want_wino:
             if args.no_tune:      # the library's untuned choices
-                wres = (L.wino_default_config(lay.shape), L.wino_prefer_fused(lay.shape), 0.0)
+                wres = (L.wino_default_config(lay.shape),
+                        "onepass" if L.wino_prefer_onepass(lay.shape) else
+                        "fused" if L.wino_prefer_fused(lay.shape) else "staged", 0.0)
             else:
                 wres = tune_layer(L, lay, V, M, (vmax, mmax))
         if want_im2col:
@@ -295,16 +316,18 @@ def main():
         else:
             use_w = wres is not None
         if use_w:
-            cfg, fused, ms = wres
+            cfg, pipe, ms = wres
             if args.pipeline != "auto":
-                fused = args.pipeline == "fused"
-            lay.algo, lay.fused = "winograd", fused
+                pipe = args.pipeline
+            lay.algo, lay.pipe = "winograd", pipe
+            if pipe == "onepass":
+                lay.setup_onepass(L)
             lay.plan = L.wino_plan(lay.shape, cfg)
             lay.U = L.alloc(lay.plan.U_bytes)
             L.wino_filter_transform(lay.plan, lay.w, lay.U)
             g = L.wino_configs()[cfg]
             log("layer %s: winograd %s, tile %dx%dx%d (cfg %d) %.3f ms%s"
-                % (lay.name(), "fused" if fused else "staged", g.bm, g.bn, g.bk, cfg, ms,
+                % (lay.name(), pipe, g.bm, g.bn, g.bk, cfg, ms,
                    " (im2col %.3f ms)" % ires[1] if ires else ""))
         else:
             cfg, ms = ires
@@ -327,7 +350,7 @@ def main():
         step()
     L.sync()
 
-    mask = {"all": 0x5f, "gemm": (1 << ST_GEMM) | (1 << 4), "none": 0}[args.stage_events]
+    mask = {"all": 0xdf, "gemm": (1 << ST_GEMM) | (1 << 4), "none": 0}[args.stage_events]
     L.timing(mask)
     L.timing_reset()
     t0 = time.perf_counter()
@@ -337,11 +360,12 @@ def main():
     elapsed = time.perf_counter() - t0
     stage = [L.stage_time(i) for i in range(4)]
     fused_stage = L.stage_time(6)
+    onepass_stage = L.stage_time(7)
     igemm_stage = L.stage_time(4)
     L.timing(0)
     if args.stage_events != "all" and not args.timed_only:
         # the other kernels: the same steps again, untimed, every kernel bracketed
-        L.timing(0x5f)
+        L.timing(0xdf)
         L.timing_reset()
         for _ in range(min(args.steps, 5)):
             step()
@@ -350,6 +374,7 @@ def main():
         for i in (ST_KT, ST_IT, ST_OT):
             stage[i] = detail[i]
         fused_stage = L.stage_time(6)
+        onepass_stage = L.stage_time(7)
         if args.stage_events == "none":
             stage[ST_GEMM] = detail[ST_GEMM]
             igemm_stage = L.stage_time(4)
@@ -361,7 +386,7 @@ def main():
 
     # dominant kernel: the batched GEMM. achieved = algorithmic flops of all its launches / their event time
     wino = [l for l in layers if l.algo == "winograd"]
-    staged = [l for l in wino if not l.fused]
+    staged = [l for l in wino if l.pipe == "staged"]
     gemm_flops_step = sum(l.algorithmic()["gemm_flops"] * l.repeats for l in staged)
     launches_step = max(1, sum(l.repeats for l in staged))
     roofline = {"kernel": "wino_gemm_kernel", "bound": "mfma", "achieved": None, "peak": PEAK_MFMA_F32_TFLOPS,
@@ -381,8 +406,8 @@ def main():
                            ("filter_transform", ST_KT, "kt_bytes")):
         ms, cnt = stage[idx]
         if cnt > 0:
-            who = staged if idx == ST_OT else wino
-            per_step = launches_step if idx == ST_OT else all_launches
+            who = staged if idx == ST_OT else ([l for l in wino if l.pipe != "onepass"] if idx == ST_IT else wino)
+            per_step = max(1, sum(l.repeats for l in who))
             b = sum(l.algorithmic()[key] * l.repeats for l in who) * (cnt / per_step)
             gbs = b / (ms * 1e-3) / 1e9
             transforms[name] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
@@ -399,6 +424,20 @@ def main():
             "unit": "GB/s", "frac": round(fbytes * k / (fused_stage[0] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
             "launches": fused_stage[1], "mfma_tflops": round(fflops * k / (fused_stage[0] * 1e-3) / 1e12, 2)}
 
+    if onepass_stage[1] > 0:
+        # one kernel reads x and U and writes y: its algorithmic bytes are those three arrays
+        ol = [l for l in wino if l.pipe == "onepass"]
+        per_step = sum(l.repeats for l in ol)
+        obytes = sum((4.0 * l.N * l.C * l.H * l.H + 256.0 * l.K * l.C + 4.0 * l.N * l.K * l.H * l.H) * l.repeats for l in ol)
+        oflops = sum(l.algorithmic()["gemm_flops"] * l.repeats for l in ol)
+        k = onepass_stage[1] / per_step
+        gbs = obytes * k / (onepass_stage[0] * 1e-3) / 1e9
+        transforms["single_kernel_conv"] = {
+            "bound": "mfma", "achieved": round(oflops * k / (onepass_stage[0] * 1e-3) / 1e12, 2),
+            "peak": PEAK_MFMA_F32_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(oflops * k / (onepass_stage[0] * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 4),
+            "launches": onepass_stage[1], "hbm_gbs": round(gbs, 1)}
+
     if igemm_stage[1] > 0:
         il = [l for l in layers if l.algo == "im2col"]
         per_step = sum(l.repeats for l in il)
@@ -413,7 +452,7 @@ def main():
 
     # per-layer detail, outside the timed region
     per_layer = []
-    L.timing(0x5f)
+    L.timing(0xdf)
     for lay in ([] if args.timed_only else layers):
         L.timing_reset()
         reps = 5
@@ -433,14 +472,17 @@ def main():
             if lay.fused:      # one kernel does the GEMM and the output transform: listed under gemm
                 st[ST_GEMM] = L.stage_time(6)[0] / reps
                 st[ST_OT] = 0.0
+            if lay.pipe == "onepass":      # one kernel does everything but the filter transform: listed under gemm
+                st[ST_GEMM] = L.stage_time(7)[0] / reps
+                st[ST_IT] = st[ST_OT] = 0.0
             total = sum(st)
             a = lay.algorithmic()
             row.update({
-                "pipeline": "fused" if lay.fused else "staged", "ms": round(total, 4),
+                "pipeline": lay.pipe, "ms": round(total, 4),
                 "gflops": round(lay.flops / (total * 1e-3) / 1e9, 1),
                 "gemm_tflops": round(a["gemm_flops"] / (st[ST_GEMM] * 1e-3) / 1e12, 2),
                 "gemm_frac_mfma": round(a["gemm_flops"] / (st[ST_GEMM] * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 3),
-                "input_tran_gbs": round(a["it_bytes"] / (st[ST_IT] * 1e-3) / 1e9, 0),
+                "input_tran_gbs": round(a["it_bytes"] / (st[ST_IT] * 1e-3) / 1e9, 0) if st[ST_IT] else None,
                 "output_tran_gbs": round(a["ot_bytes"] / (st[ST_OT] * 1e-3) / 1e9, 0) if st[ST_OT] else None,
                 "stage_ms": {"kernel_tran": round(st[ST_KT], 4), "input_tran": round(st[ST_IT], 4),
                              "gemm": round(st[ST_GEMM], 4), "output_tran": round(st[ST_OT], 4)}})
@@ -453,7 +495,7 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": args.workload, "description": desc, "batch": N, "algorithm": algo,
-                   "per_layer": ",".join("im2col" if l.algo == "im2col" else ("wino-fused" if l.fused else "wino-staged")
+                   "per_layer": ",".join("im2col" if l.algo == "im2col" else "wino-" + l.pipe
                                          for l in layers),
                    "filter_transform": "offline" if filter_ready else "online (inside the timed region)",
                    "tuned": not args.no_tune, "stage_events": args.stage_events,

@@ -91,6 +91,11 @@ _ABI = {
     "fc_wino_output_transform": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, C.c_int, _vp]),
     "fc_wino_gemm_output_fused": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, _vp, C.c_int, _vp]),
     "fc_wino_prefer_fused": (C.c_int, [C.POINTER(ConvShape)]),
+    "fc_wino_make_onepass_plan": (C.c_int, [C.POINTER(ConvShape), C.POINTER(WinoPlan)]),
+    "fc_wino_onepass_filter_transform": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp]),
+    "fc_wino_conv_onepass": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, _vp, C.c_int, _vp]),
+    "fc_wino_forward_onepass": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, _vp, C.c_int, C.c_int, _vp, _vp]),
+    "fc_wino_prefer_onepass": (C.c_int, [C.POINTER(ConvShape)]),
     "fc_wino_forward_fused": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, _vp, C.c_int, C.c_int, _vp, _vp, _vp]),
     "fc_wino_forward": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, _vp, C.c_int, C.c_int,
                                   _vp, _vp, _vp, _vp]),
@@ -283,6 +288,27 @@ class Library:
         self._check(self.c.fc_wino_forward_fused(self.ctx, C.byref(plan), x, w, bias, int(relu),
                                                  int(filter_ready), U, V, y))
 
+    # ---- the whole layer in one kernel
+    def wino_onepass_plan(self, shape):
+        plan = WinoPlan()
+        rc = self.c.fc_wino_make_onepass_plan(C.byref(shape), C.byref(plan))
+        if rc:
+            raise FastConvError(rc, self.c.fc_status_string(rc).decode())
+        return plan
+
+    def wino_onepass_filter_transform(self, plan, w, U):
+        self._check(self.c.fc_wino_onepass_filter_transform(self.ctx, C.byref(plan), w, U))
+
+    def wino_conv_onepass(self, plan, x, U, y, bias=None, relu=False):
+        self._check(self.c.fc_wino_conv_onepass(self.ctx, C.byref(plan), x, U, bias, int(relu), y))
+
+    def wino_forward_onepass(self, plan, x, w, U, y, bias=None, relu=False, filter_ready=False):
+        self._check(self.c.fc_wino_forward_onepass(self.ctx, C.byref(plan), x, w, bias, int(relu),
+                                                   int(filter_ready), U, y))
+
+    def wino_prefer_onepass(self, shape):
+        return bool(self.c.fc_wino_prefer_onepass(C.byref(shape)))
+
     def wino_forward(self, plan, x, w, U, V, M, y, bias=None, relu=False, filter_ready=False):
         self._check(self.c.fc_wino_forward(self.ctx, C.byref(plan), x, w, bias, int(relu),
                                            int(filter_ready), U, V, M, y))
@@ -307,6 +333,20 @@ class Library:
             self.wino_filter_transform(plan, dw, U)
             self.wino_input_transform(plan, dx, V)
             self.wino_gemm_output_fused(plan, U, V, y, db, relu)
+            return self.download(y, (shape.N, shape.K, plan.OH, plan.OW))
+        finally:
+            self.release(mark)
+
+    def winograd_conv_onepass(self, shape, x, w, bias=None, relu=False):
+        """Filter transform into the paired layout, then the whole layer in one kernel."""
+        plan = self.wino_onepass_plan(shape)
+        mark = self.mark()
+        try:
+            dx, dw = self.upload(x), self.upload(w)
+            db = self.upload(bias) if bias is not None else None
+            U = self.alloc(plan.U_bytes)
+            y = self.alloc(4 * shape.N * shape.K * plan.OH * plan.OW)
+            self.wino_forward_onepass(plan, dx, dw, U, y, db, relu)
             return self.download(y, (shape.N, shape.K, plan.OH, plan.OW))
         finally:
             self.release(mark)

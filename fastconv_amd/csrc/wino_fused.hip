@@ -11,35 +11,17 @@
 // global memory (L2) to registers: for reduction step (c, c+1) lane l of each
 // frequency loads U[f][c + l/32][k0 + l%32] and V[f][c + l/32][t0 + l%32], two
 // full 128-byte lines per load instruction.  Loads run three steps ahead.
-#include "fc_internal.h"
+#include "wino_fused_out.h"
 
 namespace {
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-
 struct FusedParams {
-    const float *U, *V, *bias;
-    float *y;
-    int N, K, OH, OW, relu;
-    int tH, tW;
-    long T;
+    const float *U, *V;
+    FusedOut out;
     int K_pad, C_pad;
     long T_pad;
     int nKB, nTB;
-    fc_fastdiv divTile, divTW;    // tiles per image, tiles per band
 };
-
-__device__ __forceinline__ void at6f(const float m[8], float s[6]) {
-    const float a = m[1] + m[2], b = m[1] - m[2];
-    const float c = m[3] + m[4], d = m[3] - m[4];
-    const float e = m[5] + m[6], f = m[5] - m[6];
-    s[0] = (m[0] + a) + (c + 32.0f * e);
-    s[1] = (b + 2.0f * d) + 16.0f * f;
-    s[2] = (a + 4.0f * c) + 8.0f * e;
-    s[3] = (b + 8.0f * d) + 4.0f * f;
-    s[4] = (a + 16.0f * c) + 2.0f * e;
-    s[5] = ((b + 32.0f * d) + f) + m[7];
-}
 
 // uniform base + 32-bit lane offset in bytes: the scalar-base form of global_load
 __device__ __forceinline__ float ldg(const float *base, uint32_t byteOff) {
@@ -49,10 +31,7 @@ __device__ __forceinline__ float ldg(const float *base, uint32_t byteOff) {
 constexpr int kDepth = 4;   // register slots of operand fragments (3 steps in flight + 1 in use)
 // (the offsets are 32-bit: the host checks that one frequency plane stays below 2^32 bytes)
 
-constexpr int kFW = 8;      // frequencies per wavefront
-constexpr int kThreads = 64 * (64 / kFW);
-
-__global__ __launch_bounds__(kThreads, 1) void wino_gemm_out_fused_kernel(const FusedParams p) {
+__global__ __launch_bounds__(kFusedThreads, 1) void wino_gemm_out_fused_kernel(const FusedParams p) {
     extern __shared__ __attribute__((aligned(16))) float Ml[];   // [64 f][16 k][32 t]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lrow = lane >> 5, lcol = lane & 31;
@@ -121,72 +100,8 @@ __global__ __launch_bounds__(kThreads, 1) void wino_gemm_out_fused_kernel(const 
         for (int f = 0; f < kFW; f++)
             acc[f] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u][f], bv[u][f], acc[f], 0, 0, 0);
 
-    // Output transform in two halves of 16 output channels (the LDS exchange buffer holds
-    // 64 frequencies x 16 channels x 32 tiles).  Accumulator register i of lane l is channel
-    // 8*(i/4) + 4*(l/32) + i%4, tile l%32: registers 0..7 are channels 0..15, 8..15 are 16..31.
-    const int tileN = p.tH * p.tW;
-#pragma unroll
-    for (int half = 0; half < 2; half++) {
-        if (half) __syncthreads();
-#pragma unroll
-        for (int f = 0; f < kFW; f++)
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const int krow = 8 * (i / 4) + 4 * lrow + (i % 4);
-                Ml[((wave * kFW + f) * 16 + krow) * 32 + lcol] = acc[f][half * 8 + i];
-            }
-        __syncthreads();
-        {   // one (output channel, tile) pair per thread: 16 x 32 pairs per half
-            const int krow = tid >> 5, tl = tid & 31;
-            const int k = kb * 32 + half * 16 + krow;
-            const uint32_t t = (uint32_t)tb * 32 + tl;
-            if (k < p.K && t < (uint32_t)p.T) {
-            float m[8][8];
-#pragma unroll
-            for (int f = 0; f < 64; f++) m[f >> 3][f & 7] = Ml[(f * 16 + krow) * 32 + tl];
-            float tmp[6][8];
-#pragma unroll
-            for (int jj = 0; jj < 8; jj++) {
-                const float col[8] = {m[0][jj], m[1][jj], m[2][jj], m[3][jj], m[4][jj], m[5][jj], m[6][jj], m[7][jj]};
-                float sres[6];
-                at6f(col, sres);
-#pragma unroll
-                for (int i = 0; i < 6; i++) tmp[i][jj] = sres[i];
-            }
-            const uint32_t n = fc_div(t, p.divTile), r = t - n * tileN;
-            const uint32_t th = fc_div(r, p.divTW), tw = r - th * p.tW;
-            const int rows = min(6, p.OH - (int)th * 6), cols = min(6, p.OW - (int)tw * 6);
-            const float bias = p.bias ? p.bias[k] : 0.f;
-            float *dst = p.y + (((size_t)n * p.K + k) * p.OH + (size_t)th * 6) * p.OW + tw * 6;
-            const bool pairs = cols == 6 && (p.OW & 1) == 0;    // 8-byte aligned row segments
-#pragma unroll
-            for (int i = 0; i < 6; i++) {
-                float sres[6];
-                at6f(tmp[i], sres);
-                if (i < rows) {
-#pragma unroll
-                    for (int jj = 0; jj < 6; jj++) {
-                        sres[jj] += bias;
-                        if (p.relu) sres[jj] = fmaxf(sres[jj], 0.f);
-                    }
-                    float *drow = dst + (size_t)i * p.OW;
-                    if (pairs) {
-#pragma unroll
-                        for (int jj = 0; jj < 6; jj += 2)
-                            *reinterpret_cast<float2 *>(drow + jj) = make_float2(sres[jj], sres[jj + 1]);
-                    } else {
-#pragma unroll
-                        for (int jj = 0; jj < 6; jj++)
-                            if (jj < cols) drow[jj] = sres[jj];
-                    }
-                }
-            }
-            }
-        }
-    }
+    fused_output_transform(p.out, acc, Ml, kb, tb);
 }
-
-const size_t kFusedLdsBytes = 64 * 16 * 32 * sizeof(float);   // 128 KiB
 
 }  // namespace
 
@@ -211,21 +126,17 @@ extern "C" int fc_wino_gemm_output_fused(fc_context *ctx, const fc_wino_plan *pl
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFusedLdsBytes));
         attrSet = true;
     }
-    const fc_conv_shape &s = plan->shape;
     FusedParams p;
-    p.U = U_dev; p.V = V_dev; p.bias = bias_dev; p.y = y_dev;
-    p.N = s.N; p.K = s.K; p.OH = plan->OH; p.OW = plan->OW; p.relu = relu;
-    p.tH = plan->tiles_h; p.tW = plan->tiles_w; p.T = plan->T;
+    p.U = U_dev; p.V = V_dev;
+    p.out = make_fused_out(plan, bias_dev, relu, y_dev);
     p.K_pad = plan->K_pad; p.C_pad = plan->C_pad; p.T_pad = plan->T_pad;
     p.nKB = plan->K_pad / 32;
     p.nTB = (int)((plan->T + 31) / 32);
-    p.divTile = fc_make_fastdiv((uint32_t)(p.tH * p.tW));
-    p.divTW = fc_make_fastdiv((uint32_t)p.tW);
     const long tbGroups = (p.nTB + 7) / 8;
     const long blocks = tbGroups * 8 * p.nKB;
     if (blocks >= (1l << 31)) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_gemm_output_fused: grid too large", hipSuccess);
     fc_stage_scope scope(ctx, FC_STAGE_FUSED_GEMM_OUT);
-    wino_gemm_out_fused_kernel<<<dim3((unsigned)blocks), dim3(kThreads), kFusedLdsBytes, ctx->stream>>>(p);
+    wino_gemm_out_fused_kernel<<<dim3((unsigned)blocks), dim3(kFusedThreads), kFusedLdsBytes, ctx->stream>>>(p);
     FC_LAUNCH_CHECK(ctx, "wino_gemm_out_fused_kernel");
     return FC_OK;
 }

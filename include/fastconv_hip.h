@@ -53,7 +53,8 @@ typedef enum {
     FC_STAGE_IMPLICIT_GEMM = 4,
     FC_STAGE_FILTER_PACK = 5,
     FC_STAGE_FUSED_GEMM_OUT = 6,
-    FC_STAGE_COUNT = 7
+    FC_STAGE_ONEPASS = 7,
+    FC_STAGE_COUNT = 8
 } fc_stage;
 
 typedef struct {
@@ -110,7 +111,7 @@ int fc_device_copy(fc_context *ctx, void *dst_dev, const void *src_dev, size_t b
  * 0 to switch timing off).  fc_stage_time_ms() waits for the stream, folds the
  * pending event pairs into per-stage totals and returns total milliseconds and
  * launch count since the last fc_timing_reset(). */
-#define FC_TIMING_ALL 0x7f
+#define FC_TIMING_ALL 0xff
 int fc_timing_enable(fc_context *ctx, int stage_mask);
 int fc_timing_reset(fc_context *ctx);
 int fc_stage_time_ms(fc_context *ctx, int stage, double *total_ms, long *launches);
@@ -204,6 +205,42 @@ int fc_wino_prefer_fused(const fc_conv_shape *shape);
 int fc_wino_forward_fused(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev,
                           const float *w_dev, const float *bias_dev, int relu, int filter_ready,
                           float *U_dev, float *V_dev, float *y_dev);
+
+/* ---- the whole layer in one kernel ------------------------------------ */
+
+/* gemm_config value of a plan made by fc_wino_make_onepass_plan. */
+#define FC_WINO_ONEPASS (-1)
+
+/* Plan for the single-kernel path: input transform, the 64 products and the output
+ * transform inside one workgroup per (16 tiles x 64 output channels), so neither V nor M
+ * exists (V_bytes = M_bytes = 0).  K_pad is K rounded up to 64, C_pad is C rounded up to 8.
+ * The transformed filter uses its own layout, U4[64][C_pad/4][K_pad/64][4][16][4] (channel
+ * 4q + c, output channel 64kb + 16sb + k at [f][q][kb][c][k][sb]); only
+ * fc_wino_onepass_filter_transform writes it and
+ * only fc_wino_conv_onepass reads it.  The stage calls above reject such a plan.
+ * Images narrower than 8 columns are not supported (FC_ERR_UNSUPPORTED): use the staged calls.
+ * The GPU reading of the reference's blocked pipeline taken to its end: there one block of
+ * tiles goes through input transform, TensorGEMM and output transform out of block-local
+ * scratch (winoF63/winoF63.cpp:1574-1737); here the block-local scratch is LDS and registers. */
+int fc_wino_make_onepass_plan(const fc_conv_shape *shape, fc_wino_plan *plan);
+
+/* U4 = G g G^T in the layout above (offlineKernelTransform, winoF63/winoF63.cpp:846-973). */
+int fc_wino_onepass_filter_transform(fc_context *ctx, const fc_wino_plan *plan,
+                                     const float *w_dev, float *U_dev);
+
+/* y = conv(x) (+bias, ReLU) from x and U4 in one launch. */
+int fc_wino_conv_onepass(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev,
+                         const float *U_dev, const float *bias_dev, int relu, float *y_dev);
+
+/* Filter transform (unless filter_ready) + fc_wino_conv_onepass. */
+int fc_wino_forward_onepass(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev,
+                            const float *w_dev, const float *bias_dev, int relu, int filter_ready,
+                            float *U_dev, float *y_dev);
+
+/* 1 when the single-kernel path is expected to be the fastest Winograd pipeline for this
+ * layer (measured on MI355X: 16 to 64 input channels, where the products are cheap next to
+ * moving V and M through HBM and the image is at least 8 columns wide). */
+int fc_wino_prefer_onepass(const fc_conv_shape *shape);
 
 /* All stages back to back: what winoF63_v1_single (winoF63ZC/winoF63ZC.h:5-6)
  * does in one call.  filter_ready != 0 skips the filter transform (U already

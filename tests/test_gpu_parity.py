@@ -143,6 +143,58 @@ def test_winograd_fused_full_size_layers(lib):
         assert O.max_rel_err(yf[:1], O.naive_conv_f64(sub, np.ascontiguousarray(x[:1]), w)) <= TOL_WINO
 
 
+@pytest.mark.parametrize("shp,pads", [
+    ((2, 3, 8, 11, 5), {}), ((1, 64, 56, 56, 64), {}), ((3, 10, 14, 14, 70), {}), ((2, 16, 7, 8, 33), {}),
+    ((1, 8, 30, 20, 40), {}), ((1, 3, 224, 224, 64), {}), ((4, 64, 28, 28, 128), {}), ((2, 21, 13, 13, 40), {}),
+    ((2, 6, 20, 17, 10), {"pt": 0}), ((2, 6, 20, 17, 10), {"pt": 2}), ((1, 5, 19, 23, 7), {"pt": 0, "pb": 2, "pl": 2, "pr": 0}),
+    ((5, 4, 6, 9, 4), {}), ((1, 1, 3, 8, 1), {}), ((2, 12, 50, 200, 36), {}), ((1, 2, 9, 8, 3), {"pt": 2}),
+])
+def test_winograd_single_kernel_against_oracle(lib, shp, pads):
+    """Input transform, products and output transform in one kernel (neither V nor M exists)."""
+    s = O.shape(*shp, **pads)
+    x, w = O.make_inputs(s, seed=shp[1] + 29)
+    bias = O.rng_uniform(5, (s.K,))
+    announce("single-kernel winograd", shp, pads)
+    y = lib.winograd_conv_onepass(cshape(s), x, w, bias=bias, relu=True)
+    truth = np.maximum(O.naive_conv_f64(s, x, w, bias), 0.0)
+    assert y.shape == truth.shape
+    assert O.max_rel_err(y, truth) <= TOL_WINO
+    y2 = lib.winograd_conv_onepass(cshape(s), x, w)
+    assert O.max_rel_err(y2, O.naive_conv_f64(s, x, w)) <= TOL_WINO
+
+
+def test_winograd_single_kernel_full_size_layers(lib):
+    for (N, C, H, K) in [(32, 3, 224, 64), (32, 64, 112, 128), (8, 64, 224, 64)]:
+        s = O.shape(N, C, H, H, K)
+        x, w = O.make_inputs(s, seed=2)
+        announce("single-kernel full size", (N, C, H, K))
+        yf = lib.winograd_conv_onepass(cshape(s), x, w)
+        yi = lib.implicit_gemm_conv(cshape(s), x, w)
+        assert O.max_rel_err(yf, yi) <= TOL_WINO
+        sub = O.shape(1, C, H, H, K)
+        assert O.max_rel_err(yf[-1:], O.naive_conv_f64(sub, np.ascontiguousarray(x[-1:]), w)) <= TOL_WINO
+
+
+def test_winograd_single_kernel_refuses_narrow_images(lib):
+    import fastconv_amd as F
+    with pytest.raises(F.FastConvError) as e:
+        lib.wino_onepass_plan(cshape(O.shape(1, 4, 12, 7, 4)))
+    assert e.value.status == -6
+    assert not lib.wino_prefer_onepass(cshape(O.shape(1, 4, 12, 7, 4)))
+
+
+def test_winograd_single_kernel_plan_is_not_accepted_by_the_staged_calls(lib):
+    import fastconv_amd as F
+    s = cshape(O.shape(1, 8, 12, 12, 8))
+    plan = lib.wino_onepass_plan(s)
+    assert plan.V_bytes == 0 and plan.M_bytes == 0 and plan.gemm_config == -1
+    buf = lib.alloc(1 << 20)
+    with pytest.raises(F.FastConvError):
+        lib.wino_filter_transform(plan, buf, buf)
+    with pytest.raises(F.FastConvError):
+        lib.wino_conv_onepass(lib.wino_plan(s, 0), buf, buf, buf)
+
+
 def test_winograd_rejects_unsupported(lib):
     import fastconv_amd as F
     for bad in [O.shape(1, 4, 8, 8, 4, 3, 3, 2, 2, 1), O.shape(1, 4, 8, 8, 4, 5, 5, 1, 1, 2),
