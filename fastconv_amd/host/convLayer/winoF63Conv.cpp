@@ -14,6 +14,7 @@ ConvWinoF63Layer::ConvWinoF63Layer(float *input, float *kernel, float *biasw, fl
     : ConvLayer(input, kernel, biasw, output_ref, ic, ih, iw, oc, kh, kw, sh, sw, pad_left, pad_right, pad_top,
                 pad_bottom, g, bias, nt, iter, n) {
     inputBuf = gemmBuf = kernelBuf = NULL;
+    onePass = false;
     channel_bias = NULL;
     relu = false;
     hasTail = false;
@@ -25,6 +26,8 @@ ConvWinoF63Layer::ConvWinoF63Layer(float *input, float *kernel, float *biasw, fl
     const size_t tileN = ((output_height + 5) / 6) * ((output_width + 5) / 6);
     imgBlock_best = DefaultImagesPerBlock(oc, ic, tileN, n, kCacheBudget);
     gemmConfig_best = ConvWinoF63ZCLayer::DefaultConfig(oc, ic, ih, iw, pad_top, imgBlock_best);
+    const fc_conv_shape whole = Shape((int)n);
+    if (fc_wino_prefer_onepass(&whole)) imgBlock_best = 0;      // 0: the single-kernel engine, whole batch
     enableOffKernel = 1;
     tileBlock = ocBlock = icBlock = ocRegBlock = tileRegBlock = imgBlock = 0;
 }
@@ -55,11 +58,30 @@ void ConvWinoF63Layer::SetChannelBias(const float *bias_k, bool relu_) {
 
 void ConvWinoF63Layer::SetConfig(int gemm_config, int images_per_block) {
     gemmConfig_best = gemm_config;
-    imgBlock_best = images_per_block < 1 ? 1 : (images_per_block > (int)batch ? (int)batch : images_per_block);
+    imgBlock_best = images_per_block < 0 ? 1 : (images_per_block > (int)batch ? (int)batch : images_per_block);
 }
 
 void ConvWinoF63Layer::AllocateFor(int config, int images_per_block) {
     Device &d = Device::Get();
+    onePass = images_per_block == 0;
+    if (onePass) {
+        // input transform, products and output transform in one kernel: the block-local scratch of
+        // the reference is LDS and registers, and there is no reason left to cut the batch
+        imgBlock = (int)batch;
+        hasTail = false;
+        fc_conv_shape whole = Shape(imgBlock);
+        const int orc = fc_wino_make_onepass_plan(&whole, &plan);
+        if (orc != FC_OK) {
+            fprintf(stderr, "Error: no single-kernel Winograd plan for this layer: %s\n", fc_status_string(orc));
+            exit(EXIT_FAILURE);
+        }
+        ocBlock = 64; icBlock = 4; ocRegBlock = 4; tileRegBlock = 1;
+        tileBlock = 16;
+        inputBuf = gemmBuf = NULL;
+        kernelBuf = (float *)d.Alloc(plan.U_bytes, "kernelBuf");
+        d.Check(fc_wino_onepass_filter_transform(d.ctx(), &plan, dev.kernel, kernelBuf), "fc_wino_onepass_filter_transform");
+        return;
+    }
     imgBlock = images_per_block;
     fc_conv_shape s = Shape(imgBlock);
     int rc = fc_wino_make_plan(&s, config, &plan);
@@ -88,6 +110,11 @@ void ConvWinoF63Layer::RunOnce() {
     Device &d = Device::Get();
     const size_t in_img = input_channels * input_height * input_width;
     const size_t out_img = output_channels * output_height * output_width;
+    if (onePass) {
+        d.Check(fc_wino_conv_onepass(d.ctx(), &plan, dev.input, kernelBuf, dev.bias, relu ? 1 : 0, dev.output),
+                "fc_wino_conv_onepass");
+        return;
+    }
     for (size_t n0 = 0; n0 < batch; n0 += imgBlock) {
         const fc_wino_plan *p = (n0 + imgBlock <= batch) ? &plan : &tailPlan;
         d.Check(fc_wino_forward_fused(d.ctx(), p, dev.input + n0 * in_img, dev.kernel, dev.bias, relu ? 1 : 0, 1,
@@ -115,10 +142,13 @@ int ConvWinoF63Layer::Tuning() {
 
     double minTimeusage = 1e100;
     for (int cfg = 0; cfg < fc_wino_gemm_num_configs(); cfg++) {
-        for (int ib = 1; ib <= (int)batch; ib *= 2) {
+        // images per block 0 is the single-kernel engine (no tile shape: tried once)
+        for (int ib = (cfg == 0 ? 0 : 1); ib <= (int)batch; ib = ib ? ib * 2 : 1) {
             fc_wino_plan probe;
-            fc_conv_shape ps = Shape(ib);
-            if (fc_wino_make_plan(&ps, cfg, &probe) != FC_OK) continue;
+            fc_conv_shape ps = Shape(ib ? ib : (int)batch);
+            if (ib == 0) {
+                if (fc_wino_make_onepass_plan(&ps, &probe) != FC_OK) continue;
+            } else if (fc_wino_make_plan(&ps, cfg, &probe) != FC_OK) continue;
             size_t cap, used, peak;
             fc_pool_stats(d.pool(), &cap, &used, &peak);
             if (probe.U_bytes + probe.V_bytes + 4096 > cap - used) continue;
@@ -162,19 +192,19 @@ int ConvWinoF63Layer::Init() {
     dev.Acquire(input_data, in_elems, kernel_data, output_channels * input_channels * 9, output_elements());
     if (channel_bias) dev.SetBias(channel_bias, output_channels);
     AllocateFor(gemmConfig_best, imgBlock_best);
-    printf("Algorithm: winograd F63 (blocked)\n");
+    printf("Algorithm: winograd F63 (blocked%s)\n", onePass ? ", single kernel" : "");
     printf("enableoffkernel = %d\n", enableOffKernel);
     printf("Testing ic=%zu oc=%zu width=%zu batch=%zu tileBlock=%d (%d images) ocBlock=%d icBlock=%d\n", input_channels,
            output_channels, input_width, batch, tileBlock, imgBlock, ocBlock, icBlock);
     printf("kernelBuf %zu KB\n", plan.U_bytes / 1024);
-    printf("gemmBuf   %d KB (LDS per workgroup, no device buffer)\n", 128);
+    printf("gemmBuf   %d KB (LDS per workgroup, no device buffer)\n", onePass ? 144 : 128);
     printf("inputBuf  %zu KB\n", plan.V_bytes / 1024);
     return -1;
 }
 
 int ConvWinoF63Layer::Forward() {
     Device &d = Device::Get();
-    if (!inputBuf) {
+    if (!kernelBuf) {
         fprintf(stderr, "Error: Forward() before Init()\n");
         exit(EXIT_FAILURE);
     }
@@ -190,7 +220,9 @@ int ConvWinoF63Layer::Forward() {
     d.Check(fc_timing_reset(d.ctx()), "fc_timing_reset");
     for (size_t i = 0; i < iterations; i++) RunOnce();
     // the GEMM and the output transform are one kernel here: its time is listed as TensorGEMM
-    const int stages[4] = {FC_STAGE_INPUT_TRAN, FC_STAGE_KERNEL_TRAN, FC_STAGE_FUSED_GEMM_OUT, FC_STAGE_OUTPUT_TRAN};
+    // (with the single-kernel engine that one kernel also holds the input transform)
+    const int stages[4] = {FC_STAGE_INPUT_TRAN, FC_STAGE_KERNEL_TRAN, onePass ? FC_STAGE_ONEPASS : FC_STAGE_FUSED_GEMM_OUT,
+                           FC_STAGE_OUTPUT_TRAN};
     const char *labels[4] = {"InputTran time:", "KernelTran time:", "TensorGEMM time:", "OutputTran time:"};
     for (int i = 0; i < 4; i++) {
         double ms = 0;

@@ -28,7 +28,8 @@ class ConvWinoF63Layer : public ConvLayer {
     int Forward();
 
     void SetChannelBias(const float *bias_k, bool relu);
-    // Not in the reference: fix tile shape and images per block by hand.
+    // Not in the reference: fix tile shape and images per block by hand (0 images per block: the
+    // single-kernel engine over the whole batch).
     void SetConfig(int gemm_config, int images_per_block);
     int best_config() const { return gemmConfig_best; }
     int best_images_per_block() const { return imgBlock_best; }
@@ -59,6 +60,7 @@ class ConvWinoF63Layer : public ConvLayer {
 
     fc_wino_plan plan, tailPlan;   // full blocks / the last partial block
     bool hasTail;
+    bool onePass;      // images per block 0: input transform, products and output transform in one kernel
     LayerDeviceBuffers dev;
     const float *channel_bias;
     bool relu;

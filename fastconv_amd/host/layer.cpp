@@ -33,7 +33,13 @@ int ConvolutionLayer::Init() {
     nnp_size ks = {k_, k_}, st = {s_, s_}, os = {_top_blobs[_name]->width(), _top_blobs[_name]->height()};
     const nnp_convolution_algorithm algo = select_algorithm(ks, st, os, shape_.C, oc_, shape_.N);
     winograd_ = algo == nnp_convolution_algorithm_winograd;
-    if (winograd_) {
+    onepass_ = winograd_ && fc_wino_prefer_onepass(&shape_) != 0;
+    if (onepass_) {
+        // the whole layer in one kernel: no shared scratch at all
+        d.Check(fc_wino_make_onepass_plan(&shape_, &wplan_), "fc_wino_make_onepass_plan");
+        MEMPOOL_CHECK_RETURN(private_mempool->Alloc(&U_, wplan_.U_bytes));
+        d.Check(fc_wino_onepass_filter_transform(d.ctx(), &wplan_, w_dev_, U_), "fc_wino_onepass_filter_transform");
+    } else if (winograd_) {
         d.Check(fc_wino_make_plan(&shape_, fc_wino_gemm_default_config(&shape_), &wplan_), "fc_wino_make_plan");
         fused_ = fc_wino_prefer_fused(&shape_) != 0;
         MEMPOOL_CHECK_RETURN(private_mempool->Alloc(&U_, wplan_.U_bytes));
@@ -59,6 +65,10 @@ int ConvolutionLayer::Forward() {
     const float *x = _bottom_blobs[_bottom[0]]->data();
     float *y = _top_blobs[_name]->data();
     float *scratch = NULL;
+    if (onepass_) {
+        d.Check(fc_wino_conv_onepass(d.ctx(), &wplan_, x, U_, b_dev_, relu_, y), "fc_wino_conv_onepass");
+        return 0;
+    }
     if (winograd_ || iplan_.ws_bytes) MEMPOOL_CHECK_RETURN(common_mempool->GetPtr(&scratch));
     if (winograd_) {
         float *V = scratch, *M = (float *)((char *)scratch + m_off_);

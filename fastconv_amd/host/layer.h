@@ -74,7 +74,7 @@ class ConvolutionLayer : public Layer {
     ConvolutionLayer(const std::string &name, size_t oc, size_t kernel, size_t stride, size_t pad, const float *weights,
                      const float *bias, bool relu)
         : Layer(name, "Convolution"), oc_(oc), k_(kernel), s_(stride), p_(pad), w_host_(weights), b_host_(bias),
-          relu_(relu), winograd_(false), fused_(false), w_dev_(NULL), b_dev_(NULL), U_(NULL), Wp_(NULL), table_(NULL) {}
+          relu_(relu), winograd_(false), fused_(false), onepass_(false), w_dev_(NULL), b_dev_(NULL), U_(NULL), Wp_(NULL), table_(NULL) {}
 
     int GenerateTopBlobs();
     int Init();
@@ -84,7 +84,7 @@ class ConvolutionLayer : public Layer {
    private:
     size_t oc_, k_, s_, p_;
     const float *w_host_, *b_host_;
-    bool relu_, winograd_, fused_;
+    bool relu_, winograd_, fused_, onepass_;
     float *w_dev_, *b_dev_, *U_, *Wp_;
     int32_t *table_;
     fc_conv_shape shape_;

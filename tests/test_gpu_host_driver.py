@@ -60,6 +60,20 @@ def test_tuning_writes_a_log_that_the_next_run_uses(tmp_path):
     assert len(log.read_text().strip().splitlines()) == len(set(log.read_text().strip().splitlines()))
 
 
+def test_blocked_variant_uses_the_single_kernel_engine_and_tunes(tmp_path):
+    exe = _exe("conv_test")
+    base = [exe, "-ic", "16", "-oc", "24", "-is", "28", "28", "-ks", "3", "3", "-ip", "1", "-n", "2", "-i", "2",
+            "--strict", "-a", "winograd", "--variant", "blocked"]
+    out = _run(base, cwd=str(tmp_path))
+    assert "single kernel" in out and "PASS" in out
+    out = _run(base + ["-tn", "tuning"], cwd=str(tmp_path))
+    assert "PASS" in out and "imgb=0" in out       # the single-kernel engine was among the candidates
+    # a layer outside the engine's range (8 input channels) falls back to the blocked pipeline
+    out = _run([exe, "-ic", "8", "-oc", "8", "-is", "20", "20", "-ks", "3", "3", "-i", "2", "--strict", "-a", "winograd",
+                "--variant", "blocked"], cwd=str(tmp_path))
+    assert "single kernel" not in out and "PASS" in out
+
+
 def test_layer_graph_runs_a_vgg_trunk_and_matches_the_host_chain():
     out = _run([_exe("net_test"), "-n", "2", "-is", "64", "-w", "4", "-i", "2"])
     m = re.search(r"Max relative error vs host chain: (\S+)", out)
