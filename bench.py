@@ -24,10 +24,14 @@ sys.path.insert(0, ROOT)
 
 PEAK_MFMA_F32_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch of the GEMM kernel (FETCH_SIZE + WRITE_SIZE, scaled by the copy kernel), averaged
-# over the 13 layer passes of the default workload; from profiles/vgg16_b32_winograd_hbm_traffic_pmc.txt.
-# The counters need their own rocprofv3 runs, so this is not re-measured by every bench run.
-MEASURED_GEMM_TRAFFIC = {"vgg16_b32": 485.7e6}
+# HBM bytes per launch of the GEMM kernel per layer (C, K, H) at batch 32: FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000
+# (factors from the plain copy kernel), from profiles/vgg16_b32_winograd_hbm_traffic_pmc.txt.  The counters need
+# their own rocprofv3 runs, so they are not re-measured by every bench run; `roofline.traffic` is their average
+# over the GEMM launches of a step.
+MEASURED_GEMM_TRAFFIC = {
+    32: {(128, 128, 112): 768.2e6, (128, 256, 56): 330.4e6, (256, 256, 56): 456.8e6, (256, 512, 28): 216.5e6,
+         (512, 512, 28): 327.4e6, (512, 512, 14): 173.4e6},
+}
 
 # (C, K, H, repeats): 3x3, stride 1, pad 1
 VGG16 = [(3, 64, 224, 1), (64, 64, 224, 1), (64, 128, 112, 1), (128, 128, 112, 1), (128, 256, 56, 1),
@@ -394,7 +398,9 @@ def main():
     if stage[ST_GEMM][1] > 0:
         gemm_ms, gemm_cnt = stage[ST_GEMM]
         ach = gemm_flops_step * (gemm_cnt / launches_step) / (gemm_ms * 1e-3) / 1e12
-        roofline["traffic"] = MEASURED_GEMM_TRAFFIC.get(args.workload)
+        known = MEASURED_GEMM_TRAFFIC.get(N, {})
+        if staged and all((l.C, l.K, l.H) in known for l in staged):
+            roofline["traffic"] = round(sum(known[(l.C, l.K, l.H)] * l.repeats for l in staged) / launches_step)
         roofline["algorithmic_bytes_per_launch_avg"] = round(
             sum(256.0 * (l.K * l.C + l.C * l.plan.T + l.K * l.plan.T) * l.repeats for l in staged) / launches_step)
         roofline.update(achieved=round(ach, 2), frac=round(ach / PEAK_MFMA_F32_TFLOPS, 4),

@@ -58,11 +58,13 @@ __global__ __launch_bounds__(kFusedThreads, 1) void wino_onepass_kernel(const On
     float *bounce = Vs + 2 * kVsFloats;         // [512][8]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
-    // XCD-aware order: all output-channel blocks of one tile block run back to back on one XCD,
-    // so the input patches are read from HBM once
+    // XCD-aware order (workgroup b runs on XCD b % 8): every XCD owns a contiguous range of tile
+    // blocks, so the patch rows and columns that neighbouring tiles share -- and the same patches
+    // read again by the other output-channel blocks -- are found in that XCD's L2
     const int b = blockIdx.x, xcd = b & 7, jb = b >> 3;
     const int tbl = jb / p.nKB, kb = jb - tbl * p.nKB;
-    const int tb = tbl * 8 + xcd;
+    const int perXcd = (p.nTB + 7) >> 3;
+    const int tb = xcd * perXcd + tbl;
     if (tb >= p.nTB) return;
 
     // ---- step 1: thread = row i1 of the patch of tile tl1, channel c1 of the chunk
