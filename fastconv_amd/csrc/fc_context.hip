@@ -49,6 +49,7 @@ extern "C" int fc_init(int device, fc_context **out) {
     ctx->magic = FC_CTX_MAGIC;
     ctx->device = device;
     ctx->timing_mask = 0;
+    ctx->fused_lds_granted = ctx->onepass_lds_granted = false;
     ctx->stream = nullptr;
     memset(ctx->stage_ms, 0, sizeof ctx->stage_ms);
     memset(ctx->stage_launches, 0, sizeof ctx->stage_launches);

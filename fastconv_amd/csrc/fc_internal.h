@@ -24,6 +24,8 @@ struct fc_context {
     std::vector<fc_timing_pair> pending;
     double stage_ms[FC_STAGE_COUNT];
     long stage_launches[FC_STAGE_COUNT];
+    // large dynamic LDS sizes are granted per kernel and per device, once per context
+    bool fused_lds_granted, onepass_lds_granted;
 };
 
 struct fc_pool {

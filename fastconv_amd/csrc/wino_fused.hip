@@ -120,11 +120,10 @@ extern "C" int fc_wino_gemm_output_fused(fc_context *ctx, const fc_wino_plan *pl
         return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_gemm_output_fused: padded sizes must be multiples of 32 (K, T) and 8 (C)", hipSuccess);
     if (((uintptr_t)y_dev & 7) != 0)
         return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_gemm_output_fused: y must be 8-byte aligned", hipSuccess);
-    static bool attrSet = false;
-    if (!attrSet) {
+    if (!ctx->fused_lds_granted) {
         FC_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)wino_gemm_out_fused_kernel,
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFusedLdsBytes));
-        attrSet = true;
+        ctx->fused_lds_granted = true;
     }
     FusedParams p;
     p.U = U_dev; p.V = V_dev;

@@ -359,11 +359,10 @@ extern "C" int fc_wino_conv_onepass(fc_context *ctx, const fc_wino_plan *plan, c
     if (!y_dev) return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_conv_onepass: null output", hipSuccess);
     if (((uintptr_t)y_dev & 7) != 0 || ((uintptr_t)U_dev & 15) != 0 || ((uintptr_t)x_dev & 3) != 0)
         return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_conv_onepass: y must be 8-byte and U 16-byte aligned", hipSuccess);
-    static bool attrSet = false;
-    if (!attrSet) {
+    if (!ctx->onepass_lds_granted) {
         FC_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)wino_onepass_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                               (int)kOnePassLdsBytes));
-        attrSet = true;
+        ctx->onepass_lds_granted = true;
     }
     const fc_conv_shape &s = plan->shape;
     OnePassParams p;
