@@ -119,18 +119,16 @@ __device__ __forceinline__ void gemm_tile(const float *__restrict__ U, const flo
 #pragma unroll
                 for (int ni = 0; ni < NI; ni++)
                     acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][mi], bb[cur][ni], acc[mi][ni], 0, 0, 0);
-        }
-        // scheduling: after the first MFMA of a step, issue the LDS reads of the next step,
-        // so that their latency is covered by the remaining MFMAs
-#pragma unroll
-        for (int kk = 0; kk + 2 < BK; kk += 2) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, MI + NI, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, MI * NI - 1, 0);
-        }
-        if (more) {
-            store_rows(As0 + ((s & 1) ^ 1) * (BK * BM) + aLds, ra, TL::A_ROWS * BM, SeqA());
-            store_rows(Bs0 + ((s & 1) ^ 1) * (BK * BN) + bLds, rb, TL::B_ROWS * BN, SeqB());
+            if (kk + 2 < BK) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, MI + NI, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, MI * NI - 1, 0);
+            }
+            if (kk == BK / 2 && more) {
+                // the next stage goes to the other LDS buffer half way through this one's MFMAs
+                store_rows(As0 + ((s & 1) ^ 1) * (BK * BM) + aLds, ra, TL::A_ROWS * BM, SeqA());
+                store_rows(Bs0 + ((s & 1) ^ 1) * (BK * BN) + bLds, rb, TL::B_ROWS * BN, SeqB());
+            }
         }
         __syncthreads();
     }
