@@ -407,17 +407,28 @@ def main():
                         launches=gemm_cnt, avg_launch_ms=round(gemm_ms / gemm_cnt, 5),
                         flops_per_launch_avg=gemm_flops_step / launches_step)
     transforms = {}
-    all_launches = max(1, sum(l.repeats for l in wino))
+    # online filter transforms of the staged and fused pipelines ride in the input transform's launch
+    merged = [l for l in wino if l.pipe != "onepass"] if not filter_ready else []
     for name, idx, key in (("input_transform", ST_IT, "it_bytes"), ("output_transform", ST_OT, "ot_bytes"),
                            ("filter_transform", ST_KT, "kt_bytes")):
         ms, cnt = stage[idx]
         if cnt > 0:
-            who = staged if idx == ST_OT else ([l for l in wino if l.pipe != "onepass"] if idx == ST_IT else wino)
+            if idx == ST_OT:
+                who = staged
+            elif idx == ST_IT:
+                who = [l for l in wino if l.pipe != "onepass"]
+            else:
+                who = [l for l in wino if l not in merged]
             per_step = max(1, sum(l.repeats for l in who))
-            b = sum(l.algorithmic()[key] * l.repeats for l in who) * (cnt / per_step)
+            b = sum(l.algorithmic()[key] * l.repeats for l in who)
+            if idx == ST_IT:
+                b += sum(l.algorithmic()["kt_bytes"] * l.repeats for l in merged)
+            b *= cnt / per_step
             gbs = b / (ms * 1e-3) / 1e9
             transforms[name] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                 "frac": round(gbs / PEAK_HBM_GBS, 4), "launches": cnt}
+            if idx == ST_IT and merged:
+                transforms[name]["includes"] = "filter transform (same launch)"
 
     if fused_stage[1] > 0:
         fl = [l for l in wino if l.fused]
@@ -488,7 +499,8 @@ def main():
                 "gflops": round(lay.flops / (total * 1e-3) / 1e9, 1),
                 "gemm_tflops": round(a["gemm_flops"] / (st[ST_GEMM] * 1e-3) / 1e12, 2),
                 "gemm_frac_mfma": round(a["gemm_flops"] / (st[ST_GEMM] * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 3),
-                "input_tran_gbs": round(a["it_bytes"] / (st[ST_IT] * 1e-3) / 1e9, 0) if st[ST_IT] else None,
+                "input_tran_gbs": round((a["it_bytes"] + (0 if st[ST_KT] else a["kt_bytes"])) / (st[ST_IT] * 1e-3) / 1e9, 0)
+                if st[ST_IT] else None,
                 "output_tran_gbs": round(a["ot_bytes"] / (st[ST_OT] * 1e-3) / 1e9, 0) if st[ST_OT] else None,
                 "stage_ms": {"kernel_tran": round(st[ST_KT], 4), "input_tran": round(st[ST_IT], 4),
                              "gemm": round(st[ST_GEMM], 4), "output_tran": round(st[ST_OT], 4)}})

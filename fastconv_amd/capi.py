@@ -89,6 +89,7 @@ _ABI = {
     "fc_wino_input_transform": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp]),
     "fc_wino_gemm": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, _vp]),
     "fc_wino_output_transform": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, C.c_int, _vp]),
+    "fc_wino_filter_input_transform": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, _vp, _vp]),
     "fc_wino_gemm_output_fused": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, _vp, C.c_int, _vp]),
     "fc_wino_prefer_fused": (C.c_int, [C.POINTER(ConvShape)]),
     "fc_wino_make_onepass_plan": (C.c_int, [C.POINTER(ConvShape), C.POINTER(WinoPlan)]),
@@ -217,7 +218,7 @@ class Library:
     # ---- timing
     def timing(self, on):
         """on: False/0 off, True all stages, or a bit mask of (1 << stage)."""
-        mask = 0x7f if on is True else int(on)
+        mask = 0xff if on is True else int(on)
         self._check(self.c.fc_timing_enable(self.ctx, mask))
 
     def timing_reset(self):
@@ -271,6 +272,9 @@ class Library:
 
     def wino_input_transform(self, plan, x, V):
         self._check(self.c.fc_wino_input_transform(self.ctx, C.byref(plan), x, V))
+
+    def wino_filter_input_transform(self, plan, w, U, x, V):
+        self._check(self.c.fc_wino_filter_input_transform(self.ctx, C.byref(plan), w, U, x, V))
 
     def wino_gemm(self, plan, U, V, M):
         self._check(self.c.fc_wino_gemm(self.ctx, C.byref(plan), U, V, M))

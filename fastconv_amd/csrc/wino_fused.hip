@@ -148,12 +148,8 @@ extern "C" int fc_wino_prefer_fused(const fc_conv_shape *s) {
 extern "C" int fc_wino_forward_fused(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev, const float *w_dev,
                                      const float *bias_dev, int relu, int filter_ready, float *U_dev, float *V_dev,
                                      float *y_dev) {
-    int rc;
-    if (!filter_ready) {
-        rc = fc_wino_filter_transform(ctx, plan, w_dev, U_dev);
-        if (rc) return rc;
-    }
-    rc = fc_wino_input_transform(ctx, plan, x_dev, V_dev);
+    const int rc = filter_ready ? fc_wino_input_transform(ctx, plan, x_dev, V_dev)
+                                : fc_wino_filter_input_transform(ctx, plan, w_dev, U_dev, x_dev, V_dev);
     if (rc) return rc;
     return fc_wino_gemm_output_fused(ctx, plan, U_dev, V_dev, bias_dev, relu, y_dev);
 }

@@ -13,11 +13,19 @@ namespace {
 
 // One thread per (output channel, input channel); lanes walk output channels so
 // the 64 plane stores of a wavefront are contiguous.
-__global__ __launch_bounds__(256) void wino_filter_transform_kernel(const float *__restrict__ w,
-                                                                    float *__restrict__ U, int K, int C,
-                                                                    int K_pad, int C_pad) {
-    const int k = blockIdx.x * 64 + (threadIdx.x & 63);
-    const int c = blockIdx.y * 4 + (threadIdx.x >> 6);
+struct FilterTParams {
+    const float *w;
+    float *U;
+    int K, C, K_pad, C_pad;
+};
+
+// Block (bx, by) = output channels 64*bx .. +63 of input channels 4*by .. +3.
+__device__ __forceinline__ void filter_transform_block(const FilterTParams &q, int bx, int by) {
+    const float *__restrict__ w = q.w;
+    float *__restrict__ U = q.U;
+    const int K = q.K, C = q.C, K_pad = q.K_pad, C_pad = q.C_pad;
+    const int k = bx * 64 + (threadIdx.x & 63);
+    const int c = by * 4 + (threadIdx.x >> 6);
     if (k >= K_pad || c >= C_pad) return;
     float g[3][3];
     if (k < K && c < C) {
@@ -49,6 +57,10 @@ __global__ __launch_bounds__(256) void wino_filter_transform_kernel(const float 
     }
 }
 
+__global__ __launch_bounds__(256) void wino_filter_transform_kernel(const FilterTParams q) {
+    filter_transform_block(q, blockIdx.x, blockIdx.y);
+}
+
 // ----------------------------------------------------------------- input
 
 // Tiles are numbered t = (n*tH + th)*tW + tw, so t / tW is a "band": one row of
@@ -75,12 +87,10 @@ struct InTParams {
 // tile and 8*TPB/256 of its 8 rows, and stores to the frequency planes with lanes
 // on consecutive tiles.
 template <int TPB, int ITEMS>
-__global__ __launch_bounds__(256) void wino_input_transform_kernel(const InTParams p) {
-    extern __shared__ float lds[];   // [bands][8][LW]
+__device__ __forceinline__ void input_transform_block(const InTParams &p, int bx, int c, float *lds) {
     const int tid = threadIdx.x;
-    const int c = blockIdx.y;
     const size_t plane = (size_t)p.C_pad * p.T_pad;
-    const uint32_t t0 = blockIdx.x * TPB;
+    const uint32_t t0 = bx * TPB;
     const uint32_t tLast = min((uint32_t)(t0 + TPB), (uint32_t)p.T) - 1;   // last real tile (wraps if none)
     const bool anyReal = t0 < (uint32_t)p.T;
     const uint32_t gb0 = fc_div(t0, p.divTW), gbL = anyReal ? fc_div(tLast, p.divTW) : gb0;
@@ -158,6 +168,29 @@ __global__ __launch_bounds__(256) void wino_input_transform_kernel(const InTPara
 #pragma unroll
             for (int jj = 0; jj < 8; jj++) dst[(size_t)(i * 8 + jj) * plane] = 0.f;
         }
+    }
+}
+
+template <int TPB, int ITEMS>
+__global__ __launch_bounds__(256) void wino_input_transform_kernel(const InTParams p) {
+    extern __shared__ float lds[];   // [bands][8][LW]
+    input_transform_block<TPB, ITEMS>(p, blockIdx.x, blockIdx.y, lds);
+}
+
+// Filter and input transform in one launch (the filter transform of a layer is a short
+// kernel: launched by itself it costs a launch and a drain of the whole chip per layer).
+// The first nFilter workgroups transform the filter, the others the input.
+template <int TPB, int ITEMS>
+__global__ __launch_bounds__(256) void wino_filter_input_transform_kernel(const FilterTParams q, const InTParams p,
+                                                                          int filterGridX, int nFilter, int inputGridX) {
+    extern __shared__ float lds[];
+    const int b = blockIdx.x;
+    if (b < nFilter) {
+        const int by = b / filterGridX;
+        filter_transform_block(q, b - by * filterGridX, by);
+    } else {
+        const int i = b - nFilter, c = i / inputGridX;
+        input_transform_block<TPB, ITEMS>(p, i - c * inputGridX, c, lds);
     }
 }
 
@@ -298,22 +331,28 @@ static int plan_check(fc_context *ctx, const fc_wino_plan *plan, const void *a, 
     return FC_OK;
 }
 
+static FilterTParams filter_params(const fc_wino_plan *plan, const float *w_dev, float *U_dev) {
+    FilterTParams q;
+    q.w = w_dev; q.U = U_dev;
+    q.K = plan->shape.K; q.C = plan->shape.C; q.K_pad = plan->K_pad; q.C_pad = plan->C_pad;
+    return q;
+}
+
 extern "C" int fc_wino_filter_transform(fc_context *ctx, const fc_wino_plan *plan, const float *w_dev,
                                         float *U_dev) {
     const int rc = plan_check(ctx, plan, w_dev, U_dev);
     if (rc) return rc;
     const dim3 grid((plan->K_pad + 63) / 64, (plan->C_pad + 3) / 4);
+    if (grid.y > 65535) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_filter_transform: too many channels", hipSuccess);
     fc_stage_scope scope(ctx, FC_STAGE_KERNEL_TRAN);
-    wino_filter_transform_kernel<<<grid, dim3(256), 0, ctx->stream>>>(w_dev, U_dev, plan->shape.K, plan->shape.C,
-                                                                     plan->K_pad, plan->C_pad);
+    wino_filter_transform_kernel<<<grid, dim3(256), 0, ctx->stream>>>(filter_params(plan, w_dev, U_dev));
     FC_LAUNCH_CHECK(ctx, "wino_filter_transform_kernel");
     return FC_OK;
 }
 
-extern "C" int fc_wino_input_transform(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev,
-                                       float *V_dev) {
-    const int rc = plan_check(ctx, plan, x_dev, V_dev);
-    if (rc) return rc;
+// Input transform, alone (q == NULL) or in one launch with the filter transform.
+static int launch_input_transform(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev, float *V_dev,
+                                  const FilterTParams *q) {
     const fc_conv_shape &s = plan->shape;
     InTParams p;
     p.x = x_dev; p.V = V_dev;
@@ -331,22 +370,52 @@ extern "C" int fc_wino_input_transform(fc_context *ctx, const fc_wino_plan *plan
     if (ldsBytes > 64 * 1024) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_input_transform: image too wide", hipSuccess);
     const dim3 grid((unsigned)(plan->T_pad / tpb), plan->C_pad);
     if (grid.y > 65535) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_input_transform: more than 65535 channels", hipSuccess);
-    fc_stage_scope scope(ctx, FC_STAGE_INPUT_TRAN);
     // columns (band x column pairs) per thread in pass 1
     const int itemsPerThread = (maxBands * p.LW + 255) / 256;
     if (itemsPerThread > 6) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_input_transform: image too wide", hipSuccess);
-#define FC_LAUNCH_INT(TPB_)                                                                                    \
-    do {                                                                                                       \
-        if (itemsPerThread <= 2) wino_input_transform_kernel<TPB_, 2><<<grid, dim3(256), ldsBytes, ctx->stream>>>(p);      \
-        else if (itemsPerThread <= 4) wino_input_transform_kernel<TPB_, 4><<<grid, dim3(256), ldsBytes, ctx->stream>>>(p); \
-        else wino_input_transform_kernel<TPB_, 6><<<grid, dim3(256), ldsBytes, ctx->stream>>>(p);              \
+    const int filterGridX = (plan->K_pad + 63) / 64;
+    const long nFilter = q ? (long)filterGridX * ((plan->C_pad + 3) / 4) : 0;
+    const long total = nFilter + (long)grid.x * grid.y;
+    if (total >= (1l << 31)) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_input_transform: grid too large", hipSuccess);
+    fc_stage_scope scope(ctx, FC_STAGE_INPUT_TRAN);
+#define FC_LAUNCH_ONE(TPB_, ITEMS_)                                                                                      \
+    do {                                                                                                                 \
+        if (q)                                                                                                           \
+            wino_filter_input_transform_kernel<TPB_, ITEMS_><<<dim3((unsigned)total), dim3(256), ldsBytes, ctx->stream>>>( \
+                *q, p, filterGridX, (int)nFilter, (int)grid.x);                                                          \
+        else                                                                                                             \
+            wino_input_transform_kernel<TPB_, ITEMS_><<<grid, dim3(256), ldsBytes, ctx->stream>>>(p);                    \
+    } while (0)
+#define FC_LAUNCH_INT(TPB_)                                  \
+    do {                                                     \
+        if (itemsPerThread <= 2) FC_LAUNCH_ONE(TPB_, 2);     \
+        else if (itemsPerThread <= 4) FC_LAUNCH_ONE(TPB_, 4); \
+        else FC_LAUNCH_ONE(TPB_, 6);                         \
     } while (0)
     if (tpb == 128) FC_LAUNCH_INT(128);
     else if (tpb == 64) FC_LAUNCH_INT(64);
     else FC_LAUNCH_INT(32);
 #undef FC_LAUNCH_INT
+#undef FC_LAUNCH_ONE
     FC_LAUNCH_CHECK(ctx, "wino_input_transform_kernel");
     return FC_OK;
+}
+
+extern "C" int fc_wino_input_transform(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev,
+                                       float *V_dev) {
+    const int rc = plan_check(ctx, plan, x_dev, V_dev);
+    if (rc) return rc;
+    return launch_input_transform(ctx, plan, x_dev, V_dev, NULL);
+}
+
+extern "C" int fc_wino_filter_input_transform(fc_context *ctx, const fc_wino_plan *plan, const float *w_dev, float *U_dev,
+                                              const float *x_dev, float *V_dev) {
+    int rc = plan_check(ctx, plan, w_dev, U_dev);
+    if (rc) return rc;
+    rc = plan_check(ctx, plan, x_dev, V_dev);
+    if (rc) return rc;
+    const FilterTParams q = filter_params(plan, w_dev, U_dev);
+    return launch_input_transform(ctx, plan, x_dev, V_dev, &q);
 }
 
 extern "C" int fc_wino_output_transform(fc_context *ctx, const fc_wino_plan *plan, const float *M_dev,
@@ -378,12 +447,8 @@ extern "C" int fc_wino_output_transform(fc_context *ctx, const fc_wino_plan *pla
 extern "C" int fc_wino_forward(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev, const float *w_dev,
                                const float *bias_dev, int relu, int filter_ready, float *U_dev, float *V_dev,
                                float *M_dev, float *y_dev) {
-    int rc;
-    if (!filter_ready) {
-        rc = fc_wino_filter_transform(ctx, plan, w_dev, U_dev);
-        if (rc) return rc;
-    }
-    rc = fc_wino_input_transform(ctx, plan, x_dev, V_dev);
+    int rc = filter_ready ? fc_wino_input_transform(ctx, plan, x_dev, V_dev)
+                          : fc_wino_filter_input_transform(ctx, plan, w_dev, U_dev, x_dev, V_dev);
     if (rc) return rc;
     rc = fc_wino_gemm(ctx, plan, U_dev, V_dev, M_dev);
     if (rc) return rc;

@@ -80,6 +80,16 @@ void ConvWinoF63ZCLayer::RunOnce(bool filter_ready) {
             "fc_wino_forward");
 }
 
+// The four stages as four launches (RunOnce puts the two transforms into one): used for the
+// per-stage times, which the reference prints one by one.
+void ConvWinoF63ZCLayer::RunStages(bool filter_ready) {
+    Device &d = Device::Get();
+    if (!filter_ready) d.Check(fc_wino_filter_transform(d.ctx(), &plan, dev.kernel, kernelBuf), "fc_wino_filter_transform");
+    d.Check(fc_wino_input_transform(d.ctx(), &plan, dev.input, inputBuf), "fc_wino_input_transform");
+    d.Check(fc_wino_gemm(d.ctx(), &plan, kernelBuf, inputBuf, gemmBuf), "fc_wino_gemm");
+    d.Check(fc_wino_output_transform(d.ctx(), &plan, gemmBuf, dev.bias, relu ? 1 : 0, dev.output), "fc_wino_output_transform");
+}
+
 int ConvWinoF63ZCLayer::Tuning() {
     Device &d = Device::Get();
     const fc_conv_shape s = Shape();
@@ -193,7 +203,7 @@ int ConvWinoF63ZCLayer::Forward() {
     // pass 2: the same iterations with every stage bracketed by events
     d.Check(fc_timing_enable(d.ctx(), FC_TIMING_ALL), "fc_timing_enable");
     d.Check(fc_timing_reset(d.ctx()), "fc_timing_reset");
-    for (size_t i = 0; i < iterations; i++) RunOnce(enableOffKernel != 0);
+    for (size_t i = 0; i < iterations; i++) RunStages(enableOffKernel != 0);
     const int stages[4] = {FC_STAGE_INPUT_TRAN, FC_STAGE_KERNEL_TRAN, FC_STAGE_TENSOR_GEMM, FC_STAGE_OUTPUT_TRAN};
     const char *labels[4] = {"InputTran time:", "KernelTran time:", "TensorGEMM time:", "OutputTran time:"};
     for (int i = 0; i < 4; i++) {

@@ -43,6 +43,7 @@ class ConvWinoF63ZCLayer : public ConvLayer {
     fc_conv_shape Shape() const;
     void AllocateFor(int config);
     void RunOnce(bool filter_ready);
+    void RunStages(bool filter_ready);
 
     // blocking of the GEMM stage: the chosen workgroup tile, under the names the
     // reference uses for its cache blocks

@@ -170,6 +170,14 @@ int fc_wino_filter_transform(fc_context *ctx, const fc_wino_plan *plan,
 int fc_wino_input_transform(fc_context *ctx, const fc_wino_plan *plan,
                             const float *x_dev, float *V_dev);
 
+/* Both transforms above in one launch (the filter transform of a layer is a short kernel;
+ * launched by itself it costs a launch and a drain of the chip per layer).  What the online
+ * strategy of winoF63_v1_single does back to back (winoF63ZC/winoF63ZC.cpp:433-813).  Its
+ * time is booked under FC_STAGE_INPUT_TRAN. */
+int fc_wino_filter_input_transform(fc_context *ctx, const fc_wino_plan *plan,
+                                   const float *w_dev, float *U_dev,
+                                   const float *x_dev, float *V_dev);
+
 /* M[f] = U[f]^T-layout product over input channels for all 64 frequencies in
  * one launch, on fp32 MFMA.  Replaces the depth x oc x tile loop nest calling
  * TensorGEMMInnerKernel4x4x4_v3 (winoF63ZC/winoF63ZC.cpp:818-860,

@@ -360,7 +360,32 @@ def test_stage_timers_count_launches(lib):
     lib.timing_reset()
     lib.winograd_conv(cshape(s), x, w)
     lib.winograd_conv(cshape(s), x, w)
-    for stage in range(4):
+    # the whole-layer call puts filter and input transform into one launch, booked as stage 1
+    assert lib.stage_time(0)[1] == 0
+    for stage in (1, 2, 3):
         ms, cnt = lib.stage_time(stage)
         assert cnt == 2 and ms > 0.0
+    plan = lib.wino_plan(cshape(s), 0)
+    buf = lib.alloc(max(plan.U_bytes, 4096))
+    lib.wino_filter_transform(plan, lib.upload(w), buf)
+    assert lib.stage_time(0)[1] == 1
     lib.timing(False)
+
+
+def test_filter_and_input_transform_in_one_launch_match_the_two_launches(lib):
+    for shp in [(2, 3, 8, 11, 5), (1, 64, 56, 56, 64), (3, 10, 14, 14, 70), (1, 5, 30, 200, 33)]:
+        s = cshape(O.shape(*shp))
+        x, w = O.make_inputs(O.shape(*shp), seed=5)
+        for cfg in (0, 4, 10):
+            plan = lib.wino_plan(s, cfg)
+            mark = lib.mark()
+            dx, dw = lib.upload(x), lib.upload(w)
+            U1, V1, U2, V2 = (lib.alloc(plan.U_bytes), lib.alloc(plan.V_bytes), lib.alloc(plan.U_bytes),
+                              lib.alloc(plan.V_bytes))
+            lib.wino_filter_transform(plan, dw, U1)
+            lib.wino_input_transform(plan, dx, V1)
+            lib.wino_filter_input_transform(plan, dw, U2, dx, V2)
+            ushape, vshape = (64, plan.C_pad, plan.K_pad), (64, plan.C_pad, plan.T_pad)
+            assert np.array_equal(lib.download(U1, ushape), lib.download(U2, ushape))
+            assert np.array_equal(lib.download(V1, vshape), lib.download(V2, vshape))
+            lib.release(mark)
