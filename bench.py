@@ -268,8 +268,8 @@ def main():
     if args.copy_probe:
         return copy_probe(args.copy_probe)
     if args.gpus != 1:
-        print("bench.py: this build runs on one GPU only (the layers shard by batch with no exchange step; "
-              "see DESIGN.md); run with --gpus 1", file=sys.stderr)
+        print("bench.py: this build runs on one GPU only (the layers shard by batch with no exchange step: "
+              "each GPU would hold the transformed filter and its share of the images); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
     import fastconv_amd as F
