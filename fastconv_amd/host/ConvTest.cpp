@@ -47,6 +47,7 @@ struct options {
     size_t batch;
     uint64_t seed;
     bool blocked_variant;
+    bool variant_given;
     bool check;
     bool strict;
     bool json;
@@ -70,7 +71,8 @@ void print_options_help(const char *program_name) {
         "  -i   --iterations         # iterations (default: 10)\n"
         "  -n   --batch              Images per forward pass (default: 1)\n"
         "       --seed               Seed of the input generator (default: 0)\n"
-        "       --variant            Winograd pipeline: zc (staged, default) or blocked\n"
+        "       --variant            Winograd pipeline: zc (four staged kernels) or blocked (no M buffer / single kernel);\n"
+        "                            default: whichever the library prefers for the layer\n"
         "       --no-check           Skip the naive reference and the error check\n"
         "       --strict             Exit with status 2 when the error exceeds the tolerance\n"
         "       --json               Also print one JSON line with the results\n",
@@ -125,6 +127,7 @@ struct options parse_options(int argc, char **argv) {
     options.batch = 1;
     options.seed = 0;
     options.blocked_variant = false;
+    options.variant_given = false;
     options.check = true;
     options.strict = false;
     options.json = false;
@@ -204,6 +207,7 @@ struct options parse_options(int argc, char **argv) {
                 exit(EXIT_FAILURE);
             }
             options.blocked_variant = strcmp(argv[i + 1], "blocked") == 0;
+            options.variant_given = true;
             i += 1;
         } else if (is_flag(argv[i], "--no-check", NULL)) {
             options.check = false;
@@ -355,6 +359,13 @@ int main(int argc, char *argv[]) {
         } break;
         case nnp_convolution_algorithm_winograd: {
             tolerance = 1e-3;
+            if (!options.variant_given) {
+                // few-channel layers are faster without V and M round trips through HBM
+                fc_conv_shape shp = {(int)options.batch, (int)input_channels, (int)input_size.height, (int)input_size.width,
+                                     (int)output_channels, 3, 3, 1, 1, (int)input_padding.top, (int)input_padding.bottom,
+                                     (int)input_padding.left, (int)input_padding.right};
+                options.blocked_variant = fc_wino_prefer_onepass(&shp) || fc_wino_prefer_fused(&shp);
+            }
             if (options.blocked_variant) {
                 ConvWinoF63Layer *conv = new ConvWinoF63Layer(
                     test_input, test_kernel, NULL, output_ref, input_channels, input_size.height, input_size.width,
