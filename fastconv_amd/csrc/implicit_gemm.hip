@@ -87,39 +87,35 @@ __device__ __forceinline__ void ig_store_rows(float *lds, const floatx4 (&r)[siz
 // One gathered element of the column matrix.  The row (reduction index) is the same
 // for the whole wavefront, so its table entry lives in scalar registers; the
 // per-pixel part of the bounds test is two bit masks computed once per thread.
+// The load is unconditional (an element outside the image reads the start of the image
+// instead) and its value is not touched here: whether it counts is recorded as bit `slot`
+// of `okBits` and applied when the element is written to LDS, so that the loads of a
+// stage stay in flight under the MFMAs of the stage before.
 __device__ __forceinline__ float ig_gather(const float *ximg, int pixOff, uint32_t maskR, uint32_t maskS,
-                                           const int32_t *table, int kred) {
+                                           const int32_t *table, int kred, int slot, uint32_t &okBits) {
     const int off = table[2 * kred], rs = table[2 * kred + 1];
     const bool ok = ((maskR >> (rs >> 16)) & (maskS >> (rs & 0xffff)) & 1u) != 0;
-    const float v = ximg[ok ? pixOff + off : 0];      // always an in-bounds address
-    return ok ? v : 0.f;
+    okBits |= ok ? (1u << slot) : 0u;
+    return ximg[ok ? pixOff + off : 0];
 }
 template <int... I>
-__device__ __forceinline__ void ig_gather_rows(float (&r)[sizeof...(I)], const float *ximg, int pixOff,
-                                               uint32_t maskR, uint32_t maskS, const int32_t *table, int kred0,
-                                               int rowStep, std::integer_sequence<int, I...>) {
-    ((r[I] = ig_gather(ximg, pixOff, maskR, maskS, table, kred0 + I * rowStep)), ...);
+__device__ __forceinline__ uint32_t ig_gather_rows(float (&r)[sizeof...(I)], const float *ximg, int pixOff,
+                                                   uint32_t maskR, uint32_t maskS, const int32_t *table, int kred0,
+                                                   int rowStep, std::integer_sequence<int, I...>) {
+    uint32_t okBits = 0;
+    ((r[I] = ig_gather(ximg, pixOff, maskR, maskS, table, kred0 + I * rowStep, I, okBits)), ...);
+    return okBits;
 }
 template <int... I>
-__device__ __forceinline__ void ig_scatter_rows(float *lds, const float (&r)[sizeof...(I)], int rowStride,
+__device__ __forceinline__ void ig_scatter_rows(float *lds, const float (&r)[sizeof...(I)], uint32_t okBits, int rowStride,
                                                 std::integer_sequence<int, I...>) {
-    ((lds[I * rowStride] = r[I]), ...);
+    ((lds[I * rowStride] = ((okBits >> I) & 1u) ? r[I] : 0.f), ...);
 }
 
-// Predicated 16-byte row copies for the pointwise (1x1, stride 1, no padding) case, where
-// the column matrix IS the input: row c of it is channel c of x, contiguous over the pixels.
-template <int... I>
-__device__ __forceinline__ void ig_load_rows_pw(floatx4 (&r)[sizeof...(I)], const float *p, size_t rowStride, int row0,
-                                                int rowStep, int rowLimit, bool valid,
-                                                std::integer_sequence<int, I...>) {
-    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
-    ((r[I] = (valid && row0 + I * rowStep < rowLimit) ? *reinterpret_cast<const floatx4 *>(p + (size_t)I * rowStride)
-                                                       : zero),
-     ...);
-}
-
-// PW: pointwise layers whose pixels-per-image count is a multiple of 4 copy the B tile as
-// 16-byte vectors (four pixels of one channel) instead of gathering it element by element.
+// PW: pointwise layers (1x1, stride 1, no padding: the column matrix IS the input, row c of it
+// is channel c of x, contiguous over the pixels) whose pixels-per-image count is a multiple of 4
+// and whose channel count is a multiple of BK copy the B tile as 16-byte vectors, unconditionally:
+// a pixel group past the end re-reads the last group (its columns are never stored).
 template <class TL, bool PW>
 __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmParams p) {
     constexpr int BM = TL::BM_, BN = TL::BN_, BK = TL::BK_;
@@ -165,14 +161,10 @@ __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmPara
     const int vrow = tid / (BN / 4), vcol = (tid % (BN / 4)) * 4;
     const int HW = p.H * p.W;
     const float *vg = p.x;
-    bool vvalid = false;
     if (PW) {
-        const long pix4 = (long)pb * BN + vcol;
-        vvalid = pix4 < p.Npix;
-        if (vvalid) {
-            const uint32_t n = fc_div((uint32_t)pix4, p.divOHW);
-            vg = p.x + ((size_t)n * p.C + vrow) * HW + ((uint32_t)pix4 - n * (uint32_t)HW);
-        }
+        const long pix4 = min((long)pb * BN + vcol, p.Npix - 4);
+        const uint32_t n = fc_div((uint32_t)pix4, p.divOHW);
+        vg = p.x + ((size_t)n * p.C + vrow) * HW + ((uint32_t)pix4 - n * (uint32_t)HW);
     }
     const size_t vPass = (size_t)BV_ROWS * HW, vStage = (size_t)BK * HW;
     const int vLds = vrow * BN + vcol;
@@ -182,6 +174,7 @@ __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmPara
     using SeqB = std::make_integer_sequence<int, B_LD>;
     floatx4 ra[A_LD];
     float rb[B_LD];
+    uint32_t rbOk = 0;      // bit i: rb[i] lies inside the image
     // this block's share of the reduction
     const int nStagesAll = p.Kred_pad / BK;
     const int sBegin = blockIdx.y * p.stagesPerSplit, sEnd = min(sBegin + p.stagesPerSplit, nStagesAll);
@@ -189,9 +182,9 @@ __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmPara
     ig_load_rows(ra, ag, aPass, SeqA());
     if (PW) {
         vg += (size_t)sBegin * vStage;
-        ig_load_rows_pw(rv, vg, vPass, sBegin * BK + vrow, BV_ROWS, p.C, vvalid, SeqBV());
+        ig_load_rows(rv, vg, vPass, SeqBV());
     } else {
-        ig_gather_rows(rb, ximg, pixOff, maskR, maskS, p.table, sBegin * BK + grow0, TL::ROW_STEP, SeqB());
+        rbOk = ig_gather_rows(rb, ximg, pixOff, maskR, maskS, p.table, sBegin * BK + grow0, TL::ROW_STEP, SeqB());
     }
 
     floatx16 acc[MI][NI];
@@ -204,7 +197,7 @@ __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmPara
 
     ig_store_rows(&As[0][aLds], ra, TL::A_ROWS * BM, SeqA());
     if (PW) ig_store_rows(&Bs[0][vLds], rv, BV_ROWS * BN, SeqBV());
-    else ig_scatter_rows(&Bs[0][bLds], rb, TL::ROW_STEP * BN, SeqB());
+    else ig_scatter_rows(&Bs[0][bLds], rb, rbOk, TL::ROW_STEP * BN, SeqB());
     __syncthreads();
 
     const int lrow = lane >> 5, lcol = lane & 31;
@@ -218,9 +211,9 @@ __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmPara
             ig_load_rows(ra, ag, aPass, SeqA());
             if (PW) {
                 vg += vStage;
-                ig_load_rows_pw(rv, vg, vPass, (s + 1) * BK + vrow, BV_ROWS, p.C, vvalid, SeqBV());
+                ig_load_rows(rv, vg, vPass, SeqBV());
             } else {
-                ig_gather_rows(rb, ximg, pixOff, maskR, maskS, p.table, (s + 1) * BK + grow0, TL::ROW_STEP, SeqB());
+                rbOk = ig_gather_rows(rb, ximg, pixOff, maskR, maskS, p.table, (s + 1) * BK + grow0, TL::ROW_STEP, SeqB());
             }
         }
         float a[2][MI], bb[2][NI];
@@ -246,7 +239,7 @@ __global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmPara
         if (more) {
             ig_store_rows(&As[buf ^ 1][aLds], ra, TL::A_ROWS * BM, SeqA());
             if (PW) ig_store_rows(&Bs[buf ^ 1][vLds], rv, BV_ROWS * BN, SeqBV());
-            else ig_scatter_rows(&Bs[buf ^ 1][bLds], rb, TL::ROW_STEP * BN, SeqB());
+            else ig_scatter_rows(&Bs[buf ^ 1][bLds], rb, rbOk, TL::ROW_STEP * BN, SeqB());
         }
         __syncthreads();
     }
@@ -331,7 +324,8 @@ template <class TL>
 void launch(fc_context *ctx, IgemmParams &p) {
     const dim3 grid((unsigned)(p.nKB * p.nPB), (unsigned)p.splitK);
     const bool pointwise = p.kh == 1 && p.kw == 1 && p.sh == 1 && p.sw == 1 && p.pt == 0 && p.pl == 0 &&
-                           p.OH == p.H && p.OW == p.W && (p.H * p.W) % 4 == 0 && ((uintptr_t)p.x & 15) == 0;
+                           p.OH == p.H && p.OW == p.W && (p.H * p.W) % 4 == 0 && p.C % TL::BK_ == 0 &&
+                           ((uintptr_t)p.x & 15) == 0;
     if (pointwise) igemm_conv_kernel<TL, true><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
     else igemm_conv_kernel<TL, false><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
 }
