@@ -66,6 +66,9 @@ struct IgTile {
     static constexpr int ROW_STEP = THREADS / BN;       // gather: one column, every ROW_STEP-th row
     static constexpr int B_LD = BK / ROW_STEP;
     static constexpr int LDS_BYTES = 2 * BK * (BM + BN) * 4;
+    // wavefronts per SIMD the register allocation must leave room for (the second argument of
+    // __launch_bounds__ in HIP): four for tiles up to 128x128 and the 64x256 one
+    static constexpr int MIN_WAVES = (BM * BN <= 128 * 128) ? 4 : 1;
     static_assert(THREADS % BN == 0 && BK % ROW_STEP == 0, "gather mapping");
     static_assert(BN % 64 == 0, "a wavefront gathers one row of the column matrix");
     static_assert(A_VEC % THREADS == 0 && A_LD >= 1, "every thread copies the same number of float4");
@@ -117,7 +120,7 @@ __device__ __forceinline__ void ig_scatter_rows(float *lds, const float (&r)[siz
 // and whose channel count is a multiple of BK copy the B tile as 16-byte vectors, unconditionally:
 // a pixel group past the end re-reads the last group (its columns are never stored).
 template <class TL, bool PW>
-__global__ __launch_bounds__(TL::THREADS) void igemm_conv_kernel(const IgemmParams p) {
+__global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(const IgemmParams p) {
     constexpr int BM = TL::BM_, BN = TL::BN_, BK = TL::BK_;
     constexpr int MI = TL::MI, NI = TL::NI, A_LD = TL::A_LD, B_LD = TL::B_LD;
     __shared__ __attribute__((aligned(16))) float As[2][BK * BM];
