@@ -67,8 +67,8 @@ struct IgTile {
     static constexpr int B_LD = BK / ROW_STEP;
     static constexpr int LDS_BYTES = 2 * BK * (BM + BN) * 4;
     // wavefronts per SIMD the register allocation must leave room for (the second argument of
-    // __launch_bounds__ in HIP): four for tiles up to 128x128 and the 64x256 one
-    static constexpr int MIN_WAVES = (BM * BN <= 128 * 128) ? 4 : 1;
+    // __launch_bounds__ in HIP): four for the four-wavefront tiles up to 128x128 and 64x256
+    static constexpr int MIN_WAVES = (BM * BN <= 128 * 128 && WGM * WGN == 4) ? 4 : 1;
     static_assert(THREADS % BN == 0 && BK % ROW_STEP == 0, "gather mapping");
     static_assert(BN % 64 == 0, "a wavefront gathers one row of the column matrix");
     static_assert(A_VEC % THREADS == 0 && A_LD >= 1, "every thread copies the same number of float4");
