@@ -175,6 +175,31 @@ def test_winograd_single_kernel_full_size_layers(lib):
         assert O.max_rel_err(yf[-1:], O.naive_conv_f64(sub, np.ascontiguousarray(x[-1:]), w)) <= TOL_WINO
 
 
+def test_pipelines_agree_on_random_shapes(lib):
+    """Differential check on 40 seeded random layers: implicit GEMM (the tighter path) against the
+    fp64 oracle, and the three Winograd pipelines against it."""
+    rng = np.random.default_rng(1234)
+    for case in range(40):
+        N, C, K = int(rng.integers(1, 4)), int(rng.integers(1, 41)), int(rng.integers(1, 81))
+        H, W = int(rng.integers(3, 41)), int(rng.integers(8, 41))
+        pt, pb, pl, pr = (int(v) for v in rng.integers(0, 3, size=4))
+        if H + pt + pb < 3:
+            continue
+        s = O.Shape(N, C, H, W, K, 3, 3, 1, 1, pt, pb, pl, pr)
+        cs = cshape(s)
+        x, w = O.make_inputs(s, seed=case)
+        bias = O.rng_uniform(case, (K,))
+        announce("random layer", case, (N, C, H, W, K), (pt, pb, pl, pr))
+        truth = np.maximum(O.naive_conv_f64(s, x, w, bias), 0.0)
+        yi = lib.implicit_gemm_conv(cs, x, w, bias=bias, relu=True)
+        assert O.max_rel_err(yi, truth) <= TOL_IM2COL
+        for name, y in (("staged", lib.winograd_conv(cs, x, w, bias=bias, relu=True)),
+                        ("fused", lib.winograd_conv_fused(cs, x, w, bias=bias, relu=True)),
+                        ("single kernel", lib.winograd_conv_onepass(cs, x, w, bias=bias, relu=True))):
+            assert y.shape == truth.shape, name
+            assert O.max_rel_err(y, truth) <= TOL_WINO, name
+
+
 def test_winograd_single_kernel_refuses_narrow_images(lib):
     import fastconv_amd as F
     with pytest.raises(F.FastConvError) as e:
