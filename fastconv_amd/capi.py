@@ -75,6 +75,10 @@ _ABI = {
     "fc_upload": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
     "fc_download": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
     "fc_fill_zero": (C.c_int, [_vp, _vp, C.c_size_t]),
+    "fc_graph_begin": (C.c_int, [_vp]),
+    "fc_graph_end": (C.c_int, [_vp, C.POINTER(_vp)]),
+    "fc_graph_launch": (C.c_int, [_vp, _vp]),
+    "fc_graph_destroy": (C.c_int, [_vp]),
     "fc_maxpool2x2": (C.c_int, [_vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int]),
     "fc_device_copy": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
     "fc_timing_enable": (C.c_int, [_vp, C.c_int]),
@@ -190,6 +194,11 @@ class Library:
         self._check(self.c.fc_upload(self.ctx, p, arr.ctypes.data_as(_vp), arr.nbytes))
         return p
 
+    def upload_into(self, ptr, arr):
+        """Copy a host array into device memory that was allocated before."""
+        arr = np.ascontiguousarray(arr)
+        self._check(self.c.fc_upload(self.ctx, ptr, arr.ctypes.data_as(_vp), arr.nbytes))
+
     def download(self, ptr, shape, dtype=np.float32):
         out = np.empty(shape, dtype)
         self._check(self.c.fc_download(self.ctx, out.ctypes.data_as(_vp), ptr, out.nbytes))
@@ -200,6 +209,23 @@ class Library:
 
     def device_copy(self, dst, src, nbytes):
         self._check(self.c.fc_device_copy(self.ctx, dst, src, nbytes))
+
+    # ---- recorded launch sequences
+    def graph_begin(self):
+        self._check(self.c.fc_graph_begin(self.ctx))
+
+    def graph_end(self):
+        g = _vp()
+        self._check(self.c.fc_graph_end(self.ctx, C.byref(g)))
+        return g
+
+    def graph_launch(self, g):
+        self._check(self.c.fc_graph_launch(self.ctx, g))
+
+    def graph_destroy(self, g):
+        rc = self.c.fc_graph_destroy(g)
+        if rc:
+            raise FastConvError(rc, "fc_graph_destroy")
 
     def maxpool2x2(self, x, y, N, Cc, H, W):
         self._check(self.c.fc_maxpool2x2(self.ctx, x, y, N, Cc, H, W))

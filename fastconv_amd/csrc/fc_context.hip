@@ -50,6 +50,7 @@ extern "C" int fc_init(int device, fc_context **out) {
     ctx->device = device;
     ctx->timing_mask = 0;
     ctx->fused_lds_granted = ctx->onepass_lds_granted = false;
+    ctx->capturing = false;
     ctx->stream = nullptr;
     memset(ctx->stage_ms, 0, sizeof ctx->stage_ms);
     memset(ctx->stage_launches, 0, sizeof ctx->stage_launches);
@@ -98,6 +99,7 @@ extern "C" const char *fc_last_error(fc_context *ctx) {
 
 extern "C" int fc_sync(fc_context *ctx) {
     if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    if (ctx->capturing) return fc_set_error(ctx, FC_ERR_STATE, "fc_sync: not while a graph is recorded", hipSuccess);
     FC_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
     return FC_OK;
 }
@@ -190,6 +192,7 @@ extern "C" int fc_pool_stats(fc_pool *pool, size_t *capacity, size_t *used, size
 extern "C" int fc_upload(fc_context *ctx, void *dst_dev, const void *src_host, size_t bytes) {
     if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
     if (!dst_dev || !src_host) return fc_set_error(ctx, FC_ERR_INVALID, "fc_upload: null pointer", hipSuccess);
+    if (ctx->capturing) return fc_set_error(ctx, FC_ERR_STATE, "fc_upload: not while a graph is recorded", hipSuccess);
     if (bytes == 0) return FC_OK;
     FC_HIP_CHECK(ctx, hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream));
     FC_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
@@ -199,6 +202,7 @@ extern "C" int fc_upload(fc_context *ctx, void *dst_dev, const void *src_host, s
 extern "C" int fc_download(fc_context *ctx, void *dst_host, const void *src_dev, size_t bytes) {
     if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
     if (!dst_host || !src_dev) return fc_set_error(ctx, FC_ERR_INVALID, "fc_download: null pointer", hipSuccess);
+    if (ctx->capturing) return fc_set_error(ctx, FC_ERR_STATE, "fc_download: not while a graph is recorded", hipSuccess);
     if (bytes == 0) return FC_OK;
     FC_HIP_CHECK(ctx, hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
     FC_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
@@ -267,6 +271,66 @@ extern "C" int fc_maxpool2x2(fc_context *ctx, const float *x_dev, float *y_dev, 
     return FC_OK;
 }
 
+// ---------------------------------------------------------------- graphs
+
+// A sequence of launches recorded once and replayed with one call: for layer stacks whose
+// kernels are so short that launching them one by one is what takes the time.
+extern "C" int fc_graph_begin(fc_context *ctx) {
+    if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    if (ctx->capturing) return fc_set_error(ctx, FC_ERR_STATE, "fc_graph_begin: already recording", hipSuccess);
+    if (ctx->timing_mask) return fc_set_error(ctx, FC_ERR_STATE, "fc_graph_begin: switch stage timing off first", hipSuccess);
+    FC_HIP_CHECK(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    ctx->capturing = true;
+    return FC_OK;
+}
+
+extern "C" int fc_graph_end(fc_context *ctx, fc_graph **out) {
+    if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    if (!ctx->capturing) return fc_set_error(ctx, FC_ERR_STATE, "fc_graph_end: not recording", hipSuccess);
+    ctx->capturing = false;
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
+    if (e != hipSuccess || !graph) return fc_set_error(ctx, FC_ERR_HIP, "hipStreamEndCapture", e);
+    if (!out) {
+        (void)hipGraphDestroy(graph);
+        return fc_set_error(ctx, FC_ERR_INVALID, "fc_graph_end: null output", hipSuccess);
+    }
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(graph);
+        return fc_set_error(ctx, FC_ERR_HIP, "hipGraphInstantiate", e);
+    }
+    fc_graph *g = new (std::nothrow) fc_graph();
+    if (!g) {
+        (void)hipGraphExecDestroy(exec);
+        (void)hipGraphDestroy(graph);
+        return fc_set_error(ctx, FC_ERR_OOM, "fc_graph_end", hipSuccess);
+    }
+    g->magic = FC_GRAPH_MAGIC; g->ctx = ctx; g->graph = graph; g->exec = exec;
+    *out = g;
+    return FC_OK;
+}
+
+extern "C" int fc_graph_launch(fc_context *ctx, fc_graph *g) {
+    if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    if (!g || g->magic != FC_GRAPH_MAGIC || g->ctx != ctx)
+        return fc_set_error(ctx, FC_ERR_INVALID, "fc_graph_launch: not a graph of this context", hipSuccess);
+    if (ctx->capturing) return fc_set_error(ctx, FC_ERR_STATE, "fc_graph_launch: recording", hipSuccess);
+    FC_HIP_CHECK(ctx, hipGraphLaunch(g->exec, ctx->stream));
+    return FC_OK;
+}
+
+extern "C" int fc_graph_destroy(fc_graph *g) {
+    if (!g || g->magic != FC_GRAPH_MAGIC) return FC_ERR_INVALID;
+    if (fc_ctx_ok(g->ctx)) (void)hipStreamSynchronize(g->ctx->stream);
+    (void)hipGraphExecDestroy(g->exec);
+    (void)hipGraphDestroy(g->graph);
+    g->magic = 0;
+    delete g;
+    return FC_OK;
+}
+
 // --------------------------------------------------------------- timing
 
 static int fc_timing_fold(fc_context *ctx) {
@@ -312,6 +376,8 @@ fc_stage_scope::~fc_stage_scope() {
 
 extern "C" int fc_timing_enable(fc_context *ctx, int stage_mask) {
     if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    if (ctx->capturing && stage_mask)
+        return fc_set_error(ctx, FC_ERR_STATE, "fc_timing_enable: not while a graph is recorded", hipSuccess);
     if (!stage_mask) {
         const int rc = fc_timing_fold(ctx);
         if (rc) return rc;

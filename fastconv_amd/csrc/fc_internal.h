@@ -26,6 +26,14 @@ struct fc_context {
     long stage_launches[FC_STAGE_COUNT];
     // large dynamic LDS sizes are granted per kernel and per device, once per context
     bool fused_lds_granted, onepass_lds_granted;
+    bool capturing;         // between fc_graph_begin and fc_graph_end
+};
+
+struct fc_graph {
+    uint32_t magic;
+    fc_context *ctx;
+    hipGraph_t graph;
+    hipGraphExec_t exec;
 };
 
 struct fc_pool {
@@ -37,6 +45,7 @@ struct fc_pool {
 
 static const uint32_t FC_CTX_MAGIC = 0x46434358u;   // "FCCX"
 static const uint32_t FC_POOL_MAGIC = 0x4643504cu;  // "FCPL"
+static const uint32_t FC_GRAPH_MAGIC = 0x46434752u; // "FCGR"
 
 int fc_set_error(fc_context *ctx, int status, const char *what, hipError_t err);
 bool fc_ctx_ok(const fc_context *ctx);

@@ -121,6 +121,8 @@ extern "C" int fc_wino_gemm_output_fused(fc_context *ctx, const fc_wino_plan *pl
     if (((uintptr_t)y_dev & 7) != 0)
         return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_gemm_output_fused: y must be 8-byte aligned", hipSuccess);
     if (!ctx->fused_lds_granted) {
+        if (ctx->capturing)
+            return fc_set_error(ctx, FC_ERR_STATE, "fc_wino_gemm_output_fused: run this kernel once before recording a graph with it", hipSuccess);
         FC_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)wino_gemm_out_fused_kernel,
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFusedLdsBytes));
         ctx->fused_lds_granted = true;

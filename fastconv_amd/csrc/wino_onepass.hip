@@ -360,6 +360,8 @@ extern "C" int fc_wino_conv_onepass(fc_context *ctx, const fc_wino_plan *plan, c
     if (((uintptr_t)y_dev & 7) != 0 || ((uintptr_t)U_dev & 15) != 0 || ((uintptr_t)x_dev & 3) != 0)
         return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_conv_onepass: y must be 8-byte and U 16-byte aligned", hipSuccess);
     if (!ctx->onepass_lds_granted) {
+        if (ctx->capturing)
+            return fc_set_error(ctx, FC_ERR_STATE, "fc_wino_conv_onepass: run this kernel once before recording a graph with it", hipSuccess);
         FC_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)wino_onepass_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                               (int)kOnePassLdsBytes));
         ctx->onepass_lds_granted = true;

@@ -1,7 +1,8 @@
 // Runs a VGG-16 style convolution trunk (13 x [3x3 conv + bias + ReLU], 2x2 max pooling
 // between the blocks) back to back on the device through the layer graph of layer.h, and
 // checks the result against the same chain on the host (ConvNaiveLayer + ReLU + pooling).
-//   net_test [-n batch] [-is size] [-w width_divisor] [-i iterations] [--no-check]
+//   net_test [-n batch] [-is size] [-w width_divisor] [-i iterations] [--no-check] [--graph]
+// --graph records the trunk once and replays the recording (one launch call per forward pass).
 // -w 4 divides every channel count by 4 (a small trunk whose host check takes seconds).
 #include <math.h>
 #include <stdio.h>
@@ -18,13 +19,14 @@
 
 int main(int argc, char **argv) {
     size_t batch = 1, size = 32, divisor = 4, iterations = 5;
-    bool check = true;
+    bool check = true, graph = false;
     for (int i = 1; i < argc; i++) {
         if (!strcmp(argv[i], "-n") && i + 1 < argc) batch = strtoul(argv[++i], NULL, 10);
         else if (!strcmp(argv[i], "-is") && i + 1 < argc) size = strtoul(argv[++i], NULL, 10);
         else if (!strcmp(argv[i], "-w") && i + 1 < argc) divisor = strtoul(argv[++i], NULL, 10);
         else if (!strcmp(argv[i], "-i") && i + 1 < argc) iterations = strtoul(argv[++i], NULL, 10);
         else if (!strcmp(argv[i], "--no-check")) check = false;
+        else if (!strcmp(argv[i], "--graph")) graph = true;
         else { fprintf(stderr, "Error: unknown argument '%s'\n", argv[i]); return 1; }
     }
     if (batch == 0 || size < 32 || size % 32 || divisor == 0 || 64 % divisor) {
@@ -78,6 +80,16 @@ int main(int argc, char **argv) {
     fastconv::Device &d = fastconv::Device::Get();
     net.Forward(input.data());
     d.Check(fc_sync(d.ctx()), "fc_sync");
+    if (graph) {
+        if (net.RecordGraph() != 0) return 1;
+        printf("Forward passes replay a recorded graph\n");
+        // the checked result below comes from a replay on fresh input, not from the eager pass
+        std::vector<float> other(input.size());
+        fastconv::FillUniform(2, -1.f, 1.f, other.data(), other.size());
+        net.Forward(other.data());
+        net.Forward(input.data());
+        d.Check(fc_sync(d.ctx()), "fc_sync");
+    }
     Timer t;
     t.startBench();
     for (size_t i = 0; i < iterations; i++) net.Forward(NULL);

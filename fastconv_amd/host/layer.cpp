@@ -97,7 +97,7 @@ int MaxPool2x2Layer::Forward() {
     return 0;
 }
 
-Net::Net(size_t arena_bytes) : input_(NULL) {
+Net::Net(size_t arena_bytes) : input_(NULL), graph_(NULL) {
     Device &d = Device::Get();
     arena_block_ = d.Alloc(arena_bytes, "layer graph arena");
     alloc_ = new fastconv::RangeAllocator(arena_block_, arena_bytes, 256);
@@ -105,6 +105,7 @@ Net::Net(size_t arena_bytes) : input_(NULL) {
 }
 
 Net::~Net() {
+    if (graph_) fc_graph_destroy(graph_);
     for (size_t i = 0; i < layers_.size(); i++) delete layers_[i];
     delete input_;
     delete common_;
@@ -137,8 +138,25 @@ int Net::Init() {
 
 int Net::Forward(const float *input_host) {
     if (input_host) input_->CopyData(input_host);
+    if (graph_) {
+        Device &d = Device::Get();
+        d.Check(fc_graph_launch(d.ctx(), graph_), "fc_graph_launch");
+        return 0;
+    }
     for (size_t i = 0; i < layers_.size(); i++)
         if (layers_[i]->Forward() != 0) return -1;
+    return 0;
+}
+
+int Net::RecordGraph() {
+    Device &d = Device::Get();
+    if (graph_) return 0;
+    if (Forward(NULL) != 0) return -1;      // every kernel has run once: LDS grants are in place
+    d.Check(fc_sync(d.ctx()), "fc_sync");
+    d.Check(fc_graph_begin(d.ctx()), "fc_graph_begin");
+    for (size_t i = 0; i < layers_.size(); i++)
+        if (layers_[i]->Forward() != 0) return -1;
+    d.Check(fc_graph_end(d.ctx(), &graph_), "fc_graph_end");
     return 0;
 }
 

@@ -109,6 +109,9 @@ class Net {
     void Add(Layer *layer);                 // takes ownership
     int Init();                             // GenerateTopBlobs + Init of every layer, then one common-pool Alloc
     int Forward(const float *input_host);   // upload, run all layers, no download
+    // Runs the layers once, then records them into a graph: every later Forward() replays the
+    // recording with one launch call (worth it when the kernels are short, e.g. batch 1).
+    int RecordGraph();
     const Blob<float> *output() const;
     const Blob<float> *blob_of(size_t layer) const { return layers_[layer]->top_blob((size_t)0); }
     size_t num_layers() const { return layers_.size(); }
@@ -121,6 +124,7 @@ class Net {
     Blob<float> *input_;
     std::vector<Layer *> layers_;
     void *arena_block_;
+    fc_graph *graph_;
 };
 
 }  // namespace feather

@@ -296,6 +296,21 @@ int fc_conv_implicit_gemm(fc_context *ctx, const fc_igemm_plan *plan, const floa
                           const float *Wp_dev, const int32_t *table_dev,
                           const float *bias_dev, int relu, float *ws_dev, float *y_dev);
 
+/* ---- recorded launch sequences ----------------------------------------- */
+
+/* Records every launch made on the context between fc_graph_begin and fc_graph_end into a
+ * graph that fc_graph_launch replays with one call: for stacks of layers whose kernels are
+ * so short that launching them one by one is what takes the time (batch 1).  No counterpart
+ * in the reference.  While recording, nothing runs; fc_upload, fc_download, fc_sync and
+ * stage timing are refused (FC_ERR_STATE), and the fused and single-kernel Winograd calls
+ * must have run once on the context before.  The replay reads and writes the same device
+ * buffers as the recorded calls.  fc_graph_destroy waits for the stream first. */
+typedef struct fc_graph fc_graph;
+int fc_graph_begin(fc_context *ctx);
+int fc_graph_end(fc_context *ctx, fc_graph **graph);
+int fc_graph_launch(fc_context *ctx, fc_graph *graph);
+int fc_graph_destroy(fc_graph *graph);
+
 /* ---- glue for running layers back to back ---------------------------- */
 
 /* 2x2 max pooling, stride 2, NCHW, floor((H)/2) x floor((W)/2) output: the step between

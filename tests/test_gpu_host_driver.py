@@ -81,6 +81,13 @@ def test_layer_graph_runs_a_vgg_trunk_and_matches_the_host_chain():
     assert "17 layers" in out
 
 
+def test_layer_graph_replayed_from_a_recording_matches_the_host_chain():
+    out = _run([_exe("net_test"), "-n", "1", "-is", "64", "-w", "4", "-i", "3", "--graph"])
+    m = re.search(r"Max relative error vs host chain: (\S+)", out)
+    assert "replay a recorded graph" in out
+    assert m and float(m.group(1)) <= 1e-3 and "PASS" in out
+
+
 def test_maxpool_against_numpy():
     import fastconv_amd as F
     L = F.load(0, 1 << 30)

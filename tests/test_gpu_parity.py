@@ -367,6 +367,60 @@ def test_all_ones_closed_form_full_size(lib):
     assert O.max_rel_err(yw, expect) <= TOL_WINO
 
 
+# ------------------------------------------------------- recorded sequences
+
+def test_recorded_graph_replays_match_eager_results(lib):
+    """Three layers (staged Winograd with the online filter transform, the single-kernel path,
+    an implicit GEMM that splits its reduction) recorded once; every replay, with fresh inputs and
+    eager work in between, must give the bits of the eager run on the same inputs."""
+    import fastconv_amd as F
+    s1, s2, s3 = cshape(O.shape(2, 24, 20, 20, 40)), cshape(O.shape(2, 40, 20, 20, 16)), \
+        cshape(O.Shape(2, 16, 20, 20, 48, 3, 3, 2, 2, 1, 1, 1, 1))
+    p1, p2 = lib.wino_plan(s1, 3), lib.wino_onepass_plan(s2)
+    p3 = lib.igemm_plan(s3, 0)
+    assert p3.split_k > 1
+    w1, w2, w3 = (O.rng_normal(i, shp, 0.1) for i, shp in ((1, (40, 24, 3, 3)), (2, (16, 40, 3, 3)), (3, (48, 16, 3, 3))))
+    dw1, dw2, dw3 = lib.upload(w1), lib.upload(w2), lib.upload(w3)
+    x = lib.alloc(4 * 2 * 24 * 20 * 20)
+    U1, V1, M1 = lib.alloc(p1.U_bytes), lib.alloc(p1.V_bytes), lib.alloc(p1.M_bytes)
+    y1 = lib.alloc(4 * 2 * 40 * 20 * 20)
+    U2, y2 = lib.alloc(p2.U_bytes), lib.alloc(4 * 2 * 16 * 20 * 20)
+    Wp, tab, ws = lib.alloc(p3.Wp_bytes), lib.alloc(p3.table_bytes), lib.alloc(p3.ws_bytes)
+    y3 = lib.alloc(4 * 2 * 48 * 10 * 10)
+    lib.igemm_pack_filter(p3, dw3, Wp, tab)
+
+    def run():
+        lib.wino_forward(p1, x, dw1, U1, V1, M1, y1, relu=True)
+        lib.wino_forward_onepass(p2, y1, dw2, U2, y2, relu=True)
+        lib.conv_implicit_gemm(p3, y2, Wp, tab, y3, ws=ws)
+
+    def fresh(seed):
+        lib.upload_into(x, O.rng_uniform(seed, (2, 24, 20, 20)))
+
+    fresh(10)
+    run()                       # also grants the large LDS sizes before recording
+    lib.sync()
+    lib.graph_begin()
+    with pytest.raises(F.FastConvError):
+        lib.sync()              # refused while recording
+    run()
+    g = lib.graph_end()
+    try:
+        for seed in (11, 12, 13):
+            fresh(seed)
+            run()
+            eager = lib.download(y3, (2, 48, 10, 10))
+            lib.fill_zero(y3, 4 * 2 * 48 * 10 * 10)
+            lib.fill_zero(M1, p1.M_bytes)
+            lib.sync()
+            lib.graph_launch(g)
+            replay = lib.download(y3, (2, 48, 10, 10))
+            assert np.abs(eager).max() > 0
+            assert np.array_equal(eager, replay), seed
+    finally:
+        lib.graph_destroy(g)
+
+
 # ----------------------------------------------------------------- the arena
 
 def test_pool_exhaustion_is_reported(lib):
