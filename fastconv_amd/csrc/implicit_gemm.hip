@@ -238,11 +238,19 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
 #pragma unroll
                 for (int ni = 0; ni < NI; ni++)
                     acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][mi], bb[cur][ni], acc[mi][ni], 0, 0, 0);
-        }
-        if (more) {
-            ig_store_rows(&As[buf ^ 1][aLds], ra, TL::A_ROWS * BM, SeqA());
-            if (PW) ig_store_rows(&Bs[buf ^ 1][vLds], rv, BV_ROWS * BN, SeqBV());
-            else ig_scatter_rows(&Bs[buf ^ 1][bLds], rb, rbOk, TL::ROW_STEP * BN, SeqB());
+            if (kk + 2 < BK) {
+                // after the first MFMA of a step, the LDS reads of the next step: their latency
+                // passes under the remaining MFMAs
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, MI + NI, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, MI * NI - 1, 0);
+            }
+            if (kk == BK / 2 && more) {
+                // the next stage goes to the other LDS buffer half way through this one's MFMAs
+                ig_store_rows(&As[buf ^ 1][aLds], ra, TL::A_ROWS * BM, SeqA());
+                if (PW) ig_store_rows(&Bs[buf ^ 1][vLds], rv, BV_ROWS * BN, SeqBV());
+                else ig_scatter_rows(&Bs[buf ^ 1][bLds], rb, rbOk, TL::ROW_STEP * BN, SeqB());
+            }
         }
         __syncthreads();
     }
