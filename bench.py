@@ -467,6 +467,22 @@ def main():
         roofline = dict(transforms["implicit_gemm"], kernel="igemm_conv_kernel", traffic=None,
                         avg_launch_ms=round(igemm_stage[0] / igemm_stage[1], 5))
 
+    # yardstick for the HBM-bound kernels: the library's plain copy kernel (16 bytes per lane) over the
+    # V and M scratch, outside the timed region
+    if not args.timed_only:
+        nb = int(min(vmax, mmax, 1 << 30)) // 256 * 256
+        if nb >= (64 << 20):
+            L.device_copy(M, V, nb)
+            L.sync()
+            t0c = time.perf_counter()
+            for _ in range(5):
+                L.device_copy(M, V, nb)
+            L.sync()
+            gbs = 2.0 * nb * 5 / (time.perf_counter() - t0c) / 1e9
+            transforms["copy_kernel"] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                         "frac": round(gbs / PEAK_HBM_GBS, 4), "bytes": 2 * nb,
+                                         "note": "read + write of a plain copy: what streaming kernels reach on this box"}
+
     # per-layer detail, outside the timed region
     per_layer = []
     L.timing(0xdf)
