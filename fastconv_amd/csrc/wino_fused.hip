@@ -144,7 +144,12 @@ extern "C" int fc_wino_gemm_output_fused(fc_context *ctx, const fc_wino_plan *pl
 
 extern "C" int fc_wino_prefer_fused(const fc_conv_shape *s) {
     if (!fc_shape_ok(s)) return 0;
-    return (long)s->C * s->K <= 8192 ? 1 : 0;
+    if ((long)s->C * s->K > 8192) return 0;
+    if (s->C <= 8) return 1;      // next to no products: the output transform is all there is
+    // one block of 32 tiles x 32 output channels per workgroup, one workgroup per CU at a time
+    const long OH = fc_out_dim(s->H, s->pt, s->pb, 3, 1), OW = fc_out_dim(s->W, s->pl, s->pr, 3, 1);
+    const long blocks = ((long)s->N * ((OH + 5) / 6) * ((OW + 5) / 6) + 31) / 32 * ((s->K + 31) / 32);
+    return blocks >= 512 ? 1 : 0;
 }
 
 extern "C" int fc_wino_forward_fused(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev, const float *w_dev,

@@ -261,12 +261,14 @@ extern "C" int fc_wino_gemm_get_config(int id, fc_gemm_config *cfg) {
     return FC_OK;
 }
 
-// Cost model behind the untuned choice: padded multiply-adds, divided by a relative
-// rate per tile shape (operand traffic per flop grows as (bm+bn)/(bm*bn); measured
-// on MI355X the 128x128 tile sustains the highest rate) and by how evenly the grid
-// fills the 256 CUs x 4 resident workgroups.
+// Cost model behind the untuned choice: padded multiply-adds, divided by the rate each tile
+// shape sustains relative to 128x128x16 (measured on MI355X on a layer large enough to hide
+// the grid's edges: 256 -> 256 channels at 56x56, batch 64) and by how evenly the grid fills
+// the workgroup slots of the chip.
 extern "C" int fc_wino_gemm_default_config(const fc_conv_shape *s) {
     if (!fc_shape_ok(s)) return FC_ERR_INVALID;
+    static const double kRate[] = {1.00, 0.93, 0.93, 0.89, 0.83, 0.97, 0.94, 0.945, 0.954, 0.934, 0.83};
+    static_assert(sizeof(kRate) / sizeof(kRate[0]) == sizeof(kConfigs) / sizeof(kConfigs[0]), "one rate per configuration");
     const int OH = fc_out_dim(s->H, s->pt, s->pb, 3, 1), OW = fc_out_dim(s->W, s->pl, s->pr, 3, 1);
     const double T = (double)s->N * ((OH + 5) / 6) * ((OW + 5) / 6);
     int best = 0;
@@ -275,14 +277,13 @@ extern "C" int fc_wino_gemm_default_config(const fc_conv_shape *s) {
         const fc_gemm_config &c = kConfigs[id];
         const double kp = ceil((double)s->K / c.bm) * c.bm, tp = ceil(T / c.bn) * c.bn;
         const double cp = ceil((double)s->C / c.bk) * c.bk;
-        double eff = (128.0 + 128.0) / (128.0 * 128.0) / ((double)(c.bm + c.bn) / ((double)c.bm * c.bn));
-        if (eff > 1.0) eff = 1.0;
-        if (c.bm * c.bn > 128 * 128) eff *= 0.93;      // 2 resident workgroups per CU instead of 4
-        if (c.bk == 32) eff *= 0.95;
         const double blocks = 64.0 * (kp / c.bm) * (tp / c.bn);
-        const double slots = 256.0 * (c.bm * c.bn > 128 * 128 ? 2 : 4);
-        const double fill = blocks / (ceil(blocks / slots) * slots);
-        const double cost = kp * tp * cp / (eff * (0.4 + 0.6 * fill));
+        const double slots = 256.0 * (c.bm * c.bn > 128 * 128 || c.bk == 32 ? 2 : 4);
+        // the time of a launch is nearly linear in its tile count: a partly filled last round costs
+        // little, and nothing for configuration 0, whose last round runs as quartered tiles
+        double fill = blocks / (ceil(blocks / slots) * slots);
+        if (id == 0 && blocks > slots) fill = 1.0;
+        const double cost = kp * tp * cp / (kRate[id] * (0.8 + 0.2 * fill));
         if (cost < bestCost) { bestCost = cost; best = id; }
     }
     return best;

@@ -205,7 +205,8 @@ int fc_wino_gemm_output_fused(fc_context *ctx, const fc_wino_plan *plan,
 
 /* 1 when the fused kernel is expected to beat fc_wino_gemm + fc_wino_output_transform
  * for this layer (measured on MI355X: when the transformed filter, 256*C*K bytes,
- * stays L2-resident, C*K <= 8192), else 0. */
+ * stays L2-resident, C*K <= 8192, and the layer brings at least 512 blocks of 32 tiles x 32
+ * output channels or has at most 8 input channels), else 0. */
 int fc_wino_prefer_fused(const fc_conv_shape *shape);
 
 /* Filter transform (unless filter_ready), input transform, fused GEMM + output
@@ -247,7 +248,8 @@ int fc_wino_forward_onepass(fc_context *ctx, const fc_wino_plan *plan, const flo
 
 /* 1 when the single-kernel path is expected to be the fastest Winograd pipeline for this
  * layer (measured on MI355X: 16 to 64 input channels, where the products are cheap next to
- * moving V and M through HBM and the image is at least 8 columns wide). */
+ * moving V and M through HBM, the image at least 8 columns wide, and at least 512 blocks of
+ * 16 tiles x 64 output channels, i.e. not at batch 1). */
 int fc_wino_prefer_onepass(const fc_conv_shape *shape);
 
 /* All stages back to back: what winoF63_v1_single (winoF63ZC/winoF63ZC.h:5-6)

@@ -62,8 +62,9 @@ def test_tuning_writes_a_log_that_the_next_run_uses(tmp_path):
 
 def test_blocked_variant_uses_the_single_kernel_engine_and_tunes(tmp_path):
     exe = _exe("conv_test")
-    base = [exe, "-ic", "16", "-oc", "24", "-is", "28", "28", "-ks", "3", "3", "-ip", "1", "-n", "2", "-i", "2",
-            "--strict", "-a", "winograd", "--variant", "blocked"]
+    # 32 images of 96x96: 8192 tiles, enough blocks for the library to prefer the single-kernel engine
+    base = [exe, "-ic", "16", "-oc", "24", "-is", "96", "96", "-ks", "3", "3", "-ip", "1", "-n", "32", "-i", "2",
+            "-t", "16", "--strict", "-a", "winograd", "--variant", "blocked"]
     out = _run(base, cwd=str(tmp_path))
     assert "single kernel" in out and "PASS" in out
     out = _run(base + ["-tn", "tuning"], cwd=str(tmp_path))
