@@ -351,8 +351,14 @@ extern "C" int fc_igemm_get_config(int id, fc_gemm_config *cfg) {
     return FC_OK;
 }
 
+// Untuned choice: padded multiply-adds divided by the rate each tile shape sustains relative to
+// 64x64x16 (measured on MI355X over pointwise, strided and 3x3 layers at batch 32; the shapes with
+// 128 accumulators per wavefront run one or two workgroups per CU and fall far behind) and by how
+// evenly the grid fills the chip.
 extern "C" int fc_igemm_default_config(const fc_conv_shape *s) {
     if (!fc_shape_ok(s)) return FC_ERR_INVALID;
+    static const double kRate[] = {0.93, 0.81, 0.82, 1.00, 0.75, 0.60, 0.62, 0.84};
+    static_assert(sizeof(kRate) / sizeof(kRate[0]) == sizeof(kIgConfigs) / sizeof(kIgConfigs[0]), "one rate per configuration");
     const double M = s->K, Kr = (double)s->C * s->kh * s->kw;
     const double Np = (double)s->N * fc_out_dim(s->H, s->pt, s->pb, s->kh, s->sh) * fc_out_dim(s->W, s->pl, s->pr, s->kw, s->sw);
     int best = 0;
@@ -360,13 +366,12 @@ extern "C" int fc_igemm_default_config(const fc_conv_shape *s) {
     for (int id = 0; id < kNumIgConfigs; id++) {
         const fc_gemm_config &c = kIgConfigs[id];
         const double mp = ceil(M / c.bm) * c.bm, np = ceil(Np / c.bn) * c.bn, kp = ceil(Kr / c.bk) * c.bk;
-        double eff = (128.0 + 128.0) / (128.0 * 128.0) / ((double)(c.bm + c.bn) / ((double)c.bm * c.bn));
-        if (eff > 1.0) eff = 1.0;
-        if (c.bm * c.bn > 128 * 128) eff *= 0.8;       // one resident workgroup per SIMD set
         const double blocks = (mp / c.bm) * (np / c.bn);
-        const double slots = 256.0 * (c.bm * c.bn > 128 * 128 ? 1 : 3);
-        const double fill = blocks / (ceil(blocks / slots) * slots);
-        const double cost = mp * np * kp / (eff * (0.25 + 0.75 * fill));
+        const double slots = 256.0 * (c.bm * c.bn > 128 * 128 ? 1 : 4);
+        // small layers split their reduction until about 768 workgroups exist (fc_igemm_make_plan)
+        const double eff_blocks = blocks < 512 ? 768.0 : blocks;
+        const double fill = eff_blocks / (ceil(eff_blocks / slots) * slots);
+        const double cost = mp * np * kp / (kRate[id] * (0.8 + 0.2 * fill));
         if (cost < bestCost) { bestCost = cost; best = id; }
     }
     return best;
