@@ -59,6 +59,7 @@ WORKLOADS = {
     "vgg16_b32": (_w(VGG16), 32, "winograd", "VGG-16 conv stack, 13 layers, 3x3 s1 p1, Winograd F(6,3), batch 32"),
     "vgg16_b1": (_w(VGG16), 1, "winograd", "VGG-16 conv stack, 13 layers, 3x3 s1 p1, Winograd F(6,3), batch 1"),
     "vgg16_auto_b32": (_w(VGG16), 32, "auto", "VGG-16 conv stack, faster of Winograd / implicit GEMM per layer, batch 32"),
+    "vgg16_auto_b1": (_w(VGG16), 1, "auto", "VGG-16 conv stack, faster of Winograd / implicit GEMM per layer, batch 1"),
     "resnet50_b32": (RESNET50, 32, "auto", "ResNet-50 conv layers (53 convs), auto algorithm per layer, batch 32"),
     "resnet50_b1": (RESNET50, 1, "auto", "ResNet-50 conv layers (53 convs), auto algorithm per layer, batch 1"),
     "resnet50_3x3_b32": (_w(RESNET50_3X3), 32, "winograd", "ResNet-50 3x3 s1 convs, Winograd F(6,3), batch 32"),
