@@ -28,6 +28,16 @@ __device__ __forceinline__ void store_rows(float *lds, const floatx4 (&r)[sizeof
     ((*reinterpret_cast<floatx4 *>(lds + I * rowStride) = r[I]), ...);
 }
 
+// Stages s0 .. s0+PF-1 with their register set as a compile-time constant.
+template <class F, int... U>
+__device__ __forceinline__ void stage_group(F &stage, int s0, std::integer_sequence<int, U...>) {
+    (stage(s0 + U, std::integral_constant<int, U>()), ...);
+}
+template <class F, int... U>
+__device__ __forceinline__ void stage_rest(F &stage, int s0, int nStages, std::integer_sequence<int, U...>) {
+    ((s0 + U < nStages ? stage(s0 + U, std::integral_constant<int, U>()) : (void)0), ...);
+}
+
 // Workgroup tile BM x BN x BK; WGM x WGN wavefronts, each owning
 // (BM/WGM) x (BN/WGN) of the tile as 32x32 MFMA blocks.
 template <int BM, int BN, int BK, int WGM, int WGN>
@@ -70,9 +80,18 @@ __device__ __forceinline__ void gemm_tile(const float *__restrict__ U, const flo
     using SeqA = std::make_integer_sequence<int, A_LD>;
     using SeqB = std::make_integer_sequence<int, B_LD>;
     const size_t aPass = (size_t)TL::A_ROWS * K_pad, bPass = (size_t)TL::B_ROWS * T_pad;
-    floatx4 ra[A_LD], rb[B_LD];
-    load_rows(ra, ag, aPass, SeqA());
-    load_rows(rb, bg, bPass, SeqB());
+    // Register set u holds the stages s with s % PF == u: a stage is fetched PF stages before
+    // it is parked in LDS, which is what covers the latency of L2 and HBM when a stage holds
+    // only a few MFMAs per wavefront.
+    constexpr int PF = TL::PF_;
+    const int nStages = C_pad / BK;
+    floatx4 ra[PF][A_LD], rb[PF][B_LD];
+#pragma unroll
+    for (int u = 0; u < PF; u++)
+        if (u < nStages) {
+            load_rows(ra[u], ag + (size_t)u * aStage, aPass, SeqA());
+            load_rows(rb[u], bg + (size_t)u * bStage, bPass, SeqB());
+        }
 
     floatx16 acc[MI][NI];
 #pragma unroll
@@ -82,23 +101,25 @@ __device__ __forceinline__ void gemm_tile(const float *__restrict__ U, const flo
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[mi][ni][i] = 0.f;
 
-    store_rows(As0 + aLds, ra, TL::A_ROWS * BM, SeqA());
-    store_rows(Bs0 + bLds, rb, TL::B_ROWS * BN, SeqB());
+    store_rows(As0 + aLds, ra[0], TL::A_ROWS * BM, SeqA());
+    store_rows(Bs0 + bLds, rb[0], TL::B_ROWS * BN, SeqB());
+    if (PF < nStages) {
+        load_rows(ra[0], ag + (size_t)PF * aStage, aPass, SeqA());
+        load_rows(rb[0], bg + (size_t)PF * bStage, bPass, SeqB());
+    }
     __syncthreads();
 
     // fragment addresses: lane l reads element (row kk + l/32, column base + l%32)
     const int lrow = lane >> 5, lcol = lane & 31;
     const int aFrag = lrow * BM + wm0 + lcol, bFrag = lrow * BN + wn0 + lcol;
-    const int nStages = C_pad / BK;
-    for (int s = 0; s < nStages; s++) {
-        const float *as = As0 + (s & 1) * (BK * BM), *bs = Bs0 + (s & 1) * (BK * BN);
+    // one stage: MFMAs out of LDS buffer s % 2; half way through, stage s+1 moves from register
+    // set (u+1) % PF into the other buffer and that set is refilled with stage s+1+PF
+    auto stage = [&](const int s, auto uc) __attribute__((always_inline)) {
+        constexpr int u = decltype(uc)::value;
+        const int buf = s & 1;
+        const float *as = As0 + buf * (BK * BM), *bs = Bs0 + buf * (BK * BN);
         const bool more = s + 1 < nStages;
-        if (more) {
-            ag += aStage;
-            bg += bStage;
-            load_rows(ra, ag, aPass, SeqA());
-            load_rows(rb, bg, bPass, SeqB());
-        }
+        constexpr int un = (u + 1) % PF;
         // the fragments of step kk+2 are fetched from LDS before the MFMAs of step kk are issued
         float a[2][MI], bb[2][NI];
 #pragma unroll
@@ -125,13 +146,22 @@ __device__ __forceinline__ void gemm_tile(const float *__restrict__ U, const flo
                 __builtin_amdgcn_sched_group_barrier(0x008, MI * NI - 1, 0);
             }
             if (kk == BK / 2 && more) {
-                // the next stage goes to the other LDS buffer half way through this one's MFMAs
-                store_rows(As0 + ((s & 1) ^ 1) * (BK * BM) + aLds, ra, TL::A_ROWS * BM, SeqA());
-                store_rows(Bs0 + ((s & 1) ^ 1) * (BK * BN) + bLds, rb, TL::B_ROWS * BN, SeqB());
+                // the next stage goes to the other LDS buffer half way through this one's MFMAs,
+                // and its registers are refilled with the stage PF further on
+                store_rows(As0 + (buf ^ 1) * (BK * BM) + aLds, ra[un], TL::A_ROWS * BM, SeqA());
+                store_rows(Bs0 + (buf ^ 1) * (BK * BN) + bLds, rb[un], TL::B_ROWS * BN, SeqB());
+                if (s + 1 + PF < nStages) {
+                    load_rows(ra[un], ag + (size_t)(s + 1 + PF) * aStage, aPass, SeqA());
+                    load_rows(rb[un], bg + (size_t)(s + 1 + PF) * bStage, bPass, SeqB());
+                }
             }
         }
         __syncthreads();
-    }
+    };
+    int s0 = 0;
+    for (; s0 + PF <= nStages; s0 += PF) stage_group(stage, s0, std::make_integer_sequence<int, PF>());
+    // the last nStages % PF stages
+    stage_rest(stage, s0, nStages, std::make_integer_sequence<int, PF - 1>());
 
     // D block layout: register i of lane l is row 8*(i/4) + 4*(l/32) + i%4, column l%32.
     float *Mg = M + ((size_t)f * K_pad + (size_t)kb * BM + wm0) * T_pad + (size_t)tb * BN + wn0;
@@ -195,9 +225,12 @@ __global__ __launch_bounds__(BIG::THREADS) void wino_gemm_tail_kernel(const floa
     }
 }
 
-template <int BM, int BN, int BK, int WGM, int WGN>
+// PF = register sets of global prefetch.  Measured on MI355X: 2 or 4 sets change the rate of the
+// 64x64 tile by -2..+4 % depending on the layer and cost the larger tiles a resident workgroup
+// (their register count nearly doubles), so every configuration runs with one.
+template <int BM, int BN, int BK, int WGM, int WGN, int PF = 1>
 struct TileCfg : GemmTile<BM, BN, BK, WGM, WGN> {
-    static constexpr int BM_ = BM, BN_ = BN, BK_ = BK, WGM_ = WGM, WGN_ = WGN;
+    static constexpr int BM_ = BM, BN_ = BN, BK_ = BK, WGM_ = WGM, WGN_ = WGN, PF_ = PF;
 };
 
 typedef TileCfg<128, 128, 16, 2, 2> Cfg0;
