@@ -201,6 +201,13 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
     ig_store_rows(&As[0][aLds], ra, TL::A_ROWS * BM, SeqA());
     if (PW) ig_store_rows(&Bs[0][vLds], rv, BV_ROWS * BN, SeqBV());
     else ig_scatter_rows(&Bs[0][bLds], rb, rbOk, TL::ROW_STEP * BN, SeqB());
+    // stage s of the reduction into the staging registers
+    auto load_stage = [&](const int s) __attribute__((always_inline)) {
+        ig_load_rows(ra, ag + (size_t)(s - sBegin) * aStage, aPass, SeqA());
+        if (PW) ig_load_rows(rv, vg + (size_t)(s - sBegin) * vStage, vPass, SeqBV());
+        else rbOk = ig_gather_rows(rb, ximg, pixOff, maskR, maskS, p.table, s * BK + grow0, TL::ROW_STEP, SeqB());
+    };
+    if (sBegin + 1 < sEnd) load_stage(sBegin + 1);
     __syncthreads();
 
     const int lrow = lane >> 5, lcol = lane & 31;
@@ -209,16 +216,6 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
         const int buf = (s - sBegin) & 1;
         const float *as = As[buf], *bs = Bs[buf];
         const bool more = s + 1 < sEnd;
-        if (more) {
-            ag += aStage;
-            ig_load_rows(ra, ag, aPass, SeqA());
-            if (PW) {
-                vg += vStage;
-                ig_load_rows(rv, vg, vPass, SeqBV());
-            } else {
-                rbOk = ig_gather_rows(rb, ximg, pixOff, maskR, maskS, p.table, (s + 1) * BK + grow0, TL::ROW_STEP, SeqB());
-            }
-        }
         float a[2][MI], bb[2][NI];
 #pragma unroll
         for (int mi = 0; mi < MI; mi++) a[0][mi] = as[aFrag + mi * 32];
@@ -246,10 +243,12 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
                 __builtin_amdgcn_sched_group_barrier(0x008, MI * NI - 1, 0);
             }
             if (kk == BK / 2 && more) {
-                // the next stage goes to the other LDS buffer half way through this one's MFMAs
+                // the next stage goes to the other LDS buffer half way through this one's MFMAs,
+                // and the one after it is requested at once: a whole stage in flight
                 ig_store_rows(&As[buf ^ 1][aLds], ra, TL::A_ROWS * BM, SeqA());
                 if (PW) ig_store_rows(&Bs[buf ^ 1][vLds], rv, BV_ROWS * BN, SeqBV());
                 else ig_scatter_rows(&Bs[buf ^ 1][bLds], rb, rbOk, TL::ROW_STEP * BN, SeqB());
+                if (s + 2 < sEnd) load_stage(s + 2);
             }
         }
         __syncthreads();
