@@ -400,8 +400,14 @@ extern "C" int fc_igemm_make_plan(const fc_conv_shape *s, int config, fc_igemm_p
     const long blocks = (long)(plan->K_pad / cfg.bm) * ((npix + cfg.bn - 1) / cfg.bn);
     const int stages = plan->Kred_pad / cfg.bk;
     int split = 1;
-    if (blocks < 512) {
-        split = (int)((768 + blocks - 1) / blocks);
+    // A grid of two to four workgroups per CU is placed unevenly by the dispatcher (some CUs get
+    // one more than their share and set the time of the launch): with a long reduction, splitting
+    // it to about six per CU is worth the second pass (measured: 3x3 stride-2 layers of ResNet-50
+    // at batch 32 -9 %, 2048 -> 512 at 7x7 -6 %; with a short reduction the second pass costs more).
+    const bool longReduction = stages >= 64;
+    const long below = longReduction ? 1024 : 512, target = longReduction ? 1536 : 768;
+    if (blocks < below) {
+        split = (int)((target + blocks - 1) / blocks);
         if (split > stages / 4) split = stages / 4;
         if (split > 32) split = 32;
         if (split < 1) split = 1;
