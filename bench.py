@@ -386,6 +386,24 @@ def main():
         L.timing(0)
 
     ms_per_step = elapsed / args.steps * 1e3
+    # shader clock under this workload: the same steps once more, untimed, beside the library's
+    # clock probe (the published MFMA peak is quoted at the maximum clock; power management runs
+    # the shaders slower under fp32 MFMA load with real data)
+    shader_clock = None
+    if not args.timed_only:
+        n_probe = max(3, min(args.steps, 10))
+        samples = 64
+        sample_us = int(min(100000, max(20, ms_per_step * 1e3 * n_probe / samples)))
+        step()
+        step()
+        L.clock_probe_begin(samples, sample_us)
+        for _ in range(n_probe + 1):
+            step()
+        L.sync()
+        mhz = L.clock_probe_end()
+        shader_clock = {"nominal_mhz": None, "mean_mhz": round(sum(mhz) / len(mhz), 1), "min_mhz": round(min(mhz), 1),
+                        "max_mhz": round(max(mhz), 1), "samples": len(mhz), "sample_us": sample_us,
+                        "over": "%d more steps of the same workload, untimed" % n_probe}
     step_flops = sum(l.flops * l.repeats for l in layers)
     value = step_flops / (ms_per_step * 1e-3) / 1e9
 
@@ -407,6 +425,10 @@ def main():
         roofline.update(achieved=round(ach, 2), frac=round(ach / PEAK_MFMA_F32_TFLOPS, 4),
                         launches=gemm_cnt, avg_launch_ms=round(gemm_ms / gemm_cnt, 5),
                         flops_per_launch_avg=gemm_flops_step / launches_step)
+        if shader_clock:
+            # 256 CUs x 256 fp32 MFMA flops per clock: what the measured clock allows
+            at_clock = info["compute_units"] * 256 * shader_clock["mean_mhz"] * 1e6 / 1e12
+            roofline.update(peak_at_measured_clock=round(at_clock, 1), frac_at_measured_clock=round(ach / at_clock, 4))
     transforms = {}
     # online filter transforms of the staged and fused pipelines ride in the input transform's launch
     merged = [l for l in wino if l.pipe != "onepass"] if not filter_ready else []
@@ -536,11 +558,14 @@ def main():
                    "tuned": not args.no_tune, "stage_events": args.stage_events,
                    "device": info["arch"], "compute_units": info["compute_units"], "clock_mhz": info["clock_mhz"]},
         "roofline": roofline,
+        "shader_clock": shader_clock,
         "transform_rooflines": transforms,
         "layers": per_layer,
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
+    if shader_clock:
+        shader_clock["nominal_mhz"] = info["clock_mhz"]
     L.close()
     print(json.dumps(out), flush=True)
 

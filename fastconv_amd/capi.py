@@ -84,6 +84,8 @@ _ABI = {
     "fc_timing_enable": (C.c_int, [_vp, C.c_int]),
     "fc_timing_reset": (C.c_int, [_vp]),
     "fc_stage_time_ms": (C.c_int, [_vp, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_long)]),
+    "fc_clock_probe_begin": (C.c_int, [_vp, C.c_int, C.c_int]),
+    "fc_clock_probe_end": (C.c_int, [_vp, C.POINTER(C.c_double), C.c_int, C.POINTER(C.c_int)]),
     "fc_wino_gemm_num_configs": (C.c_int, []),
     "fc_wino_gemm_get_config": (C.c_int, [C.c_int, C.POINTER(GemmConfig)]),
     "fc_wino_gemm_default_config": (C.c_int, [C.POINTER(ConvShape)]),
@@ -254,6 +256,17 @@ class Library:
         ms, cnt = C.c_double(), C.c_long()
         self._check(self.c.fc_stage_time_ms(self.ctx, stage, C.byref(ms), C.byref(cnt)))
         return ms.value, cnt.value
+
+    def clock_probe_begin(self, samples, sample_us):
+        """Start sampling the shader clock beside whatever is enqueued next."""
+        self._check(self.c.fc_clock_probe_begin(self.ctx, samples, sample_us))
+
+    def clock_probe_end(self):
+        """Wait for the probe; shader clock of every sample in MHz."""
+        buf = (C.c_double * 256)()
+        n = C.c_int()
+        self._check(self.c.fc_clock_probe_end(self.ctx, buf, 256, C.byref(n)))
+        return [buf[i] for i in range(min(n.value, 256))]
 
     # ---- configs / plans
     def wino_configs(self):

@@ -52,6 +52,9 @@ extern "C" int fc_init(int device, fc_context **out) {
     ctx->fused_lds_granted = ctx->onepass_lds_granted = false;
     ctx->capturing = false;
     ctx->stream = nullptr;
+    ctx->probe_stream = nullptr;
+    ctx->probe_buf = nullptr;
+    ctx->probe_samples = 0;
     memset(ctx->stage_ms, 0, sizeof ctx->stage_ms);
     memset(ctx->stage_launches, 0, sizeof ctx->stage_launches);
     if (hipGetDeviceProperties(&ctx->props, device) != hipSuccess) { delete ctx; return FC_ERR_NO_DEVICE; }
@@ -72,9 +75,64 @@ extern "C" int fc_destroy(fc_context *ctx) {
     (void)hipStreamSynchronize(ctx->stream);
     for (auto &p : ctx->pending) { (void)hipEventDestroy(p.start); (void)hipEventDestroy(p.stop); }
     for (auto &ev : ctx->free_events) (void)hipEventDestroy(ev);
+    if (ctx->probe_stream) {
+        (void)hipStreamSynchronize(ctx->probe_stream);
+        (void)hipStreamDestroy(ctx->probe_stream);
+    }
+    if (ctx->probe_buf) (void)hipFree(ctx->probe_buf);
     (void)hipStreamDestroy(ctx->stream);
     ctx->magic = 0;
     delete ctx;
+    return FC_OK;
+}
+
+// One lane: per sample, wait on the constant 100 MHz counter and record both counters' advance.
+// The wait is bounded twice: by the real-time counter, and by a cap on the number of polls.
+__global__ __launch_bounds__(64) void fc_clock_probe_kernel(unsigned long long *out, int samples,
+                                                            unsigned long long ticksPerSample) {
+    if (threadIdx.x != 0) return;
+    for (int i = 0; i < samples; i++) {
+        const unsigned long long r0 = wall_clock64(), c0 = clock64();
+        unsigned long long r1 = r0;
+        for (int poll = 0; poll < (1 << 22) && r1 - r0 < ticksPerSample; poll++) {
+            __builtin_amdgcn_s_sleep(8);
+            r1 = wall_clock64();
+        }
+        const unsigned long long c1 = clock64();
+        out[2 * i] = r1 - r0;
+        out[2 * i + 1] = c1 - c0;
+    }
+}
+
+static const int kProbeMaxSamples = 256;
+
+extern "C" int fc_clock_probe_begin(fc_context *ctx, int samples, int sample_us) {
+    if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    if (samples < 1 || samples > kProbeMaxSamples || sample_us < 1 || sample_us > 100000)
+        return fc_set_error(ctx, FC_ERR_INVALID, "fc_clock_probe_begin: 1..256 samples of 1..100000 us", hipSuccess);
+    if (ctx->capturing) return fc_set_error(ctx, FC_ERR_STATE, "fc_clock_probe_begin: a graph is being recorded", hipSuccess);
+    if (ctx->probe_samples) return fc_set_error(ctx, FC_ERR_STATE, "fc_clock_probe_begin: a probe is already running", hipSuccess);
+    FC_HIP_CHECK(ctx, hipSetDevice(ctx->device));
+    if (!ctx->probe_stream) FC_HIP_CHECK(ctx, hipStreamCreateWithFlags(&ctx->probe_stream, hipStreamNonBlocking));
+    if (!ctx->probe_buf) FC_HIP_CHECK(ctx, hipMalloc((void **)&ctx->probe_buf, kProbeMaxSamples * 2 * sizeof(unsigned long long)));
+    fc_clock_probe_kernel<<<dim3(1), dim3(64), 0, ctx->probe_stream>>>(ctx->probe_buf, samples, 100ull * sample_us);
+    FC_LAUNCH_CHECK(ctx, "fc_clock_probe_kernel");
+    ctx->probe_samples = samples;
+    return FC_OK;
+}
+
+extern "C" int fc_clock_probe_end(fc_context *ctx, double *mhz, int capacity, int *n_samples) {
+    if (!fc_ctx_ok(ctx)) return FC_ERR_STATE;
+    if (!mhz || capacity < 1 || !n_samples) return fc_set_error(ctx, FC_ERR_INVALID, "fc_clock_probe_end: null or empty output", hipSuccess);
+    if (!ctx->probe_samples) return fc_set_error(ctx, FC_ERR_STATE, "fc_clock_probe_end: no probe is running", hipSuccess);
+    const int n = ctx->probe_samples;
+    ctx->probe_samples = 0;
+    FC_HIP_CHECK(ctx, hipStreamSynchronize(ctx->probe_stream));
+    unsigned long long host[kProbeMaxSamples * 2];
+    FC_HIP_CHECK(ctx, hipMemcpy(host, ctx->probe_buf, (size_t)n * 2 * sizeof(unsigned long long), hipMemcpyDeviceToHost));
+    *n_samples = n;
+    for (int i = 0; i < n && i < capacity; i++)
+        mhz[i] = host[2 * i] ? (double)host[2 * i + 1] * 100.0 / (double)host[2 * i] : 0.0;     // ticks of 10 ns
     return FC_OK;
 }
 

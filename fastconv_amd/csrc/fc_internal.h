@@ -27,6 +27,10 @@ struct fc_context {
     // large dynamic LDS sizes are granted per kernel and per device, once per context
     bool fused_lds_granted, onepass_lds_granted;
     bool capturing;         // between fc_graph_begin and fc_graph_end
+    // shader-clock probe: its own stream and result buffer, created on first use
+    hipStream_t probe_stream;
+    unsigned long long *probe_buf;
+    int probe_samples;      // > 0 while a probe is running
 };
 
 struct fc_graph {

@@ -116,6 +116,19 @@ int fc_timing_enable(fc_context *ctx, int stage_mask);
 int fc_timing_reset(fc_context *ctx);
 int fc_stage_time_ms(fc_context *ctx, int stage, double *total_ms, long *launches);
 
+/* Shader clock under load.  The published MFMA peak is quoted at the maximum shader clock
+ * (2400 MHz on MI355X); under fp32 MFMA load with real data the chip's power management runs
+ * the shaders slower, and the clock it sustains is what bounds the products.
+ * fc_clock_probe_begin starts a one-wavefront kernel on a stream of its own that, `samples`
+ * times (1..256), waits `sample_us` microseconds (1..100000) on the constant 100 MHz counter and
+ * records how far the shader-clock counter moved meanwhile; work enqueued through this context
+ * afterwards runs beside it.  fc_clock_probe_end waits for the probe and returns the shader
+ * clock of every sample in MHz (at most `capacity` of them; *n_samples = how many were taken).
+ * One probe at a time per context; not while a graph is being recorded.  No counterpart in the
+ * reference, whose Timer (utility/helper.cpp:113-148) sees wall time only. */
+int fc_clock_probe_begin(fc_context *ctx, int samples, int sample_us);
+int fc_clock_probe_end(fc_context *ctx, double *mhz, int capacity, int *n_samples);
+
 /* ---- Winograd F(6x6,3x3), stride 1 ------------------------------------ */
 
 /* Tile shapes of the batched GEMM stage.  The reference tunes

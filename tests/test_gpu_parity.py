@@ -451,6 +451,29 @@ def test_stage_timers_count_launches(lib):
     lib.timing(False)
 
 
+def test_clock_probe_reports_a_plausible_shader_clock(lib):
+    import fastconv_amd as F
+    s = O.shape(4, 64, 56, 56, 64)
+    x, w = O.make_inputs(s, seed=2)
+    ref = lib.winograd_conv(cshape(s), x, w)
+    with pytest.raises(F.FastConvError):
+        lib.clock_probe_end()                   # nothing running
+    with pytest.raises(F.FastConvError):
+        lib.clock_probe_begin(0, 100)
+    with pytest.raises(F.FastConvError):
+        lib.clock_probe_begin(8, 0)
+    lib.clock_probe_begin(12, 200)
+    with pytest.raises(F.FastConvError):
+        lib.clock_probe_begin(4, 100)           # one at a time
+    y = lib.winograd_conv(cshape(s), x, w)      # work beside the probe is not disturbed
+    mhz = lib.clock_probe_end()
+    announce("shader clock samples (MHz):", [round(v) for v in mhz])
+    assert len(mhz) == 12 and all(300.0 < v < 3000.0 for v in mhz)
+    np.testing.assert_array_equal(y, ref)
+    lib.clock_probe_begin(2, 50)                # usable again
+    assert len(lib.clock_probe_end()) == 2
+
+
 def test_filter_and_input_transform_in_one_launch_match_the_two_launches(lib):
     for shp in [(2, 3, 8, 11, 5), (1, 64, 56, 56, 64), (3, 10, 14, 14, 70), (1, 5, 30, 200, 33)]:
         s = cshape(O.shape(*shp))
