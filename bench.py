@@ -29,8 +29,8 @@ PEAK_HBM_GBS = 8000.0
 # their own rocprofv3 runs, so they are not re-measured by every bench run; `roofline.traffic` is their average
 # over the GEMM launches of a step.
 MEASURED_GEMM_TRAFFIC = {
-    32: {(128, 128, 112): 768.2e6, (128, 256, 56): 330.4e6, (256, 256, 56): 456.8e6, (256, 512, 28): 216.5e6,
-         (512, 512, 28): 327.4e6, (512, 512, 14): 173.4e6},
+    32: {(128, 128, 112): 768.1e6, (128, 256, 56): 330.4e6, (256, 256, 56): 456.2e6, (256, 512, 28): 197.2e6,
+         (512, 512, 28): 289.7e6, (512, 512, 14): 155.1e6},
 }
 
 # (C, K, H, repeats): 3x3, stride 1, pad 1
