@@ -51,6 +51,7 @@ struct IgemmParams {
     int nKB, nPB;
     int splitK, stagesPerSplit;   // reduction split over blockIdx.y; partial sums go to ws
     float *ws;                    // [splitK][K][Npix] when splitK > 1
+    int fastStore;                // K is a whole number of tiles, every output byte offset fits 32 bits, bias 16-byte aligned
     fc_fastdiv divOHW, divOW;
 };
 
@@ -254,9 +255,57 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
         __syncthreads();
     }
 
-    // epilogue: column = pixel (lane%32), rows = output channels
+    // epilogue: column = pixel (lane%32), rows = output channels.  Register i of an accumulator
+    // block is row 8*(i/4) + 4*(lane/32) + i%4: element (row r, column c) of the tile goes to
+    // dst[colOff(c) + (rowBase + r) * rowStride], with dst = y (colOff = n*K*OHW + pixel in image,
+    // rowStride = OHW) or the partial-sum slab of this split (colOff = pixel, rowStride = Npix).
     const int OHW = p.OH * p.OW;
-    if (p.splitK > 1) {
+    const bool partial = p.splitK > 1;
+    const int rowBase = kb * BM + wm0 + 4 * lrow;
+    if (p.fastStore) {
+        // every row of the tile is a real output channel and every byte offset fits 32 bits: a
+        // scalar base, one 32-bit offset per store, no predicates
+        char *dst = reinterpret_cast<char *>(partial ? p.ws : p.y);
+        const uint32_t rowStride = 4u * (partial ? (uint32_t)p.Npix : (uint32_t)OHW);      // bytes
+        const uint32_t slab = partial ? (uint32_t)blockIdx.y * (uint32_t)p.K * (uint32_t)p.Npix : 0u;
+        const bool plain = partial || (p.bias == nullptr && !p.relu);
+#pragma unroll
+        for (int ni = 0; ni < NI; ni++) {
+            const long opix = (long)pb * BN + wn0 + ni * 32 + lcol;
+            if (opix >= p.Npix) continue;
+            uint32_t off;
+            if (partial) {
+                off = slab + (uint32_t)opix;
+            } else {
+                const uint32_t n = fc_div((uint32_t)opix, p.divOHW);
+                off = n * (uint32_t)p.K * (uint32_t)OHW + ((uint32_t)opix - n * (uint32_t)OHW);
+            }
+            off = 4u * off + (uint32_t)rowBase * rowStride;
+            if (plain) {
+#pragma unroll
+                for (int mi = 0; mi < MI; mi++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++)
+                        *reinterpret_cast<float *>(dst + (off + (uint32_t)(mi * 32 + 8 * (i / 4) + (i % 4)) * rowStride)) = acc[mi][ni][i];
+            } else {
+#pragma unroll
+                for (int mi = 0; mi < MI; mi++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        floatx4 bq = {0.f, 0.f, 0.f, 0.f};
+                        if (p.bias) bq = *reinterpret_cast<const floatx4 *>(p.bias + rowBase + mi * 32 + 8 * q);
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            float v = acc[mi][ni][q * 4 + j] + bq[j];
+                            if (p.relu) v = fmaxf(v, 0.f);
+                            *reinterpret_cast<float *>(dst + (off + (uint32_t)(mi * 32 + 8 * q + j) * rowStride)) = v;
+                        }
+                    }
+            }
+        }
+        return;
+    }
+    if (partial) {
         // partial sums, [split][k][pixel]; igemm_reduce_kernel adds them up in split order
         float *wz = p.ws + (size_t)blockIdx.y * p.K * p.Npix;
 #pragma unroll
@@ -267,7 +316,7 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
             for (int mi = 0; mi < MI; mi++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) {
-                    const int k = kb * BM + wm0 + mi * 32 + 8 * (i / 4) + 4 * lrow + (i % 4);
+                    const int k = rowBase + mi * 32 + 8 * (i / 4) + (i % 4);
                     if (k < p.K) wz[(size_t)k * p.Npix + opix] = acc[mi][ni][i];
                 }
         }
@@ -284,7 +333,7 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
         for (int mi = 0; mi < MI; mi++)
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                const int k = kb * BM + wm0 + mi * 32 + 8 * (i / 4) + 4 * lrow + (i % 4);
+                const int k = rowBase + mi * 32 + 8 * (i / 4) + (i % 4);
                 if (k < p.K) {
                     float v = acc[mi][ni][i];
                     if (p.bias) v += p.bias[k];
@@ -470,6 +519,8 @@ extern "C" int fc_conv_implicit_gemm(fc_context *ctx, const fc_igemm_plan *plan,
     p.splitK = plan->split_k;
     p.stagesPerSplit = ((plan->Kred_pad / cfg.bk) + plan->split_k - 1) / plan->split_k;
     p.ws = ws_dev;
+    p.fastStore = s.K % cfg.bm == 0 && 4.0 * s.N * s.K * plan->OH * plan->OW < 4294967296.0 &&
+                  4.0 * plan->split_k * s.K * (double)plan->Npix < 4294967296.0 && ((uintptr_t)bias_dev & 15) == 0;
     if ((long)p.nKB * p.nPB >= (1l << 31)) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_conv_implicit_gemm: grid too large", hipSuccess);
     fc_stage_scope scope(ctx, FC_STAGE_IMPLICIT_GEMM);
     switch (plan->config) {
