@@ -273,6 +273,25 @@ def test_implicit_gemm_every_tile_config(lib):
         assert O.max_rel_err(y, truth) <= TOL_IM2COL, cfg.id
 
 
+def test_implicit_gemm_full_tile_epilogue_paths(lib):
+    """Output-channel counts that are whole tiles take the predicate-free epilogue (plain, and
+    with bias / ReLU); pixel blocks that straddle images and end inside a block are part of it."""
+    for shp in [(3, 32, 13, 13, 256, 1, 1, 1, 1, 0), (2, 48, 17, 17, 256, 3, 3, 2, 2, 1), (5, 64, 14, 14, 256, 1, 1, 1, 1, 0)]:
+        s = O.shape(*shp)
+        x, w = O.make_inputs(s, seed=8)
+        bias = O.rng_uniform(12, (s.K,))
+        plain = O.naive_conv_f64(s, x, w)
+        with_bias = np.maximum(O.naive_conv_f64(s, x, w, bias), 0.0)
+        only_bias = O.naive_conv_f64(s, x, w, bias)
+        for cfg in lib.igemm_configs():
+            announce("full-tile epilogue", shp, "tile", cfg.bm, cfg.bn)
+            assert O.max_rel_err(lib.implicit_gemm_conv(cshape(s), x, w, config=cfg.id), plain) <= TOL_IM2COL
+            assert O.max_rel_err(lib.implicit_gemm_conv(cshape(s), x, w, bias=bias, relu=True, config=cfg.id),
+                                 with_bias) <= TOL_IM2COL
+            assert O.max_rel_err(lib.implicit_gemm_conv(cshape(s), x, w, bias=bias, config=cfg.id),
+                                 only_bias) <= TOL_IM2COL
+
+
 def test_implicit_gemm_split_reduction_is_exact_and_repeatable(lib):
     """Batch-1 layers are too small to fill the GPU: their reduction is split and the parts
     are added in a fixed order, so two runs give the same bits."""
