@@ -95,33 +95,42 @@ __device__ __forceinline__ void ig_store_rows(float *lds, const floatx4 (&r)[siz
 // instead) and its value is not touched here: whether it counts is recorded as bit `slot`
 // of `okBits` and applied when the element is written to LDS, so that the loads of a
 // stage stay in flight under the MFMAs of the stage before.
+// MASKED = false: every tap of every output pixel lies inside the image (no padding on the top
+// and left, and the last window ends inside) and the reduction has no padding rows: no test.
+template <bool MASKED>
 __device__ __forceinline__ float ig_gather(const float *ximg, int pixOff, uint32_t maskR, uint32_t maskS,
                                            const int32_t *table, int kred, int slot, uint32_t &okBits) {
-    const int off = table[2 * kred], rs = table[2 * kred + 1];
+    const int off = table[2 * kred];
+    if (!MASKED) return ximg[pixOff + off];
+    const int rs = table[2 * kred + 1];
     const bool ok = ((maskR >> (rs >> 16)) & (maskS >> (rs & 0xffff)) & 1u) != 0;
     okBits |= ok ? (1u << slot) : 0u;
     return ximg[ok ? pixOff + off : 0];
 }
-template <int... I>
+template <bool MASKED, int... I>
 __device__ __forceinline__ uint32_t ig_gather_rows(float (&r)[sizeof...(I)], const float *ximg, int pixOff,
                                                    uint32_t maskR, uint32_t maskS, const int32_t *table, int kred0,
                                                    int rowStep, std::integer_sequence<int, I...>) {
     uint32_t okBits = 0;
-    ((r[I] = ig_gather(ximg, pixOff, maskR, maskS, table, kred0 + I * rowStep, I, okBits)), ...);
+    ((r[I] = ig_gather<MASKED>(ximg, pixOff, maskR, maskS, table, kred0 + I * rowStep, I, okBits)), ...);
     return okBits;
 }
-template <int... I>
+template <bool MASKED, int... I>
 __device__ __forceinline__ void ig_scatter_rows(float *lds, const float (&r)[sizeof...(I)], uint32_t okBits, int rowStride,
                                                 std::integer_sequence<int, I...>) {
-    ((lds[I * rowStride] = ((okBits >> I) & 1u) ? r[I] : 0.f), ...);
+    ((lds[I * rowStride] = (!MASKED || ((okBits >> I) & 1u)) ? r[I] : 0.f), ...);
 }
+
+// How the B tile (a slice of the column matrix) reaches LDS.
+enum { IG_GATHER = 0, IG_POINTWISE = 1, IG_GATHER_INSIDE = 2 };
 
 // PW: pointwise layers (1x1, stride 1, no padding: the column matrix IS the input, row c of it
 // is channel c of x, contiguous over the pixels) whose pixels-per-image count is a multiple of 4
 // and whose channel count is a multiple of BK copy the B tile as 16-byte vectors, unconditionally:
 // a pixel group past the end re-reads the last group (its columns are never stored).
-template <class TL, bool PW>
+template <class TL, int MODE>
 __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(const IgemmParams p) {
+    constexpr bool PW = MODE == IG_POINTWISE, MASKED = MODE != IG_GATHER_INSIDE;
     constexpr int BM = TL::BM_, BN = TL::BN_, BK = TL::BK_;
     constexpr int MI = TL::MI, NI = TL::NI, A_LD = TL::A_LD, B_LD = TL::B_LD;
     __shared__ __attribute__((aligned(16))) float As[2][BK * BM];
@@ -188,7 +197,7 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
         vg += (size_t)sBegin * vStage;
         ig_load_rows(rv, vg, vPass, SeqBV());
     } else {
-        rbOk = ig_gather_rows(rb, ximg, pixOff, maskR, maskS, p.table, sBegin * BK + grow0, TL::ROW_STEP, SeqB());
+        rbOk = ig_gather_rows<MASKED>(rb, ximg, pixOff, maskR, maskS, p.table, sBegin * BK + grow0, TL::ROW_STEP, SeqB());
     }
 
     floatx16 acc[MI][NI];
@@ -201,12 +210,12 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
 
     ig_store_rows(&As[0][aLds], ra, TL::A_ROWS * BM, SeqA());
     if (PW) ig_store_rows(&Bs[0][vLds], rv, BV_ROWS * BN, SeqBV());
-    else ig_scatter_rows(&Bs[0][bLds], rb, rbOk, TL::ROW_STEP * BN, SeqB());
+    else ig_scatter_rows<MASKED>(&Bs[0][bLds], rb, rbOk, TL::ROW_STEP * BN, SeqB());
     // stage s of the reduction into the staging registers
     auto load_stage = [&](const int s) __attribute__((always_inline)) {
         ig_load_rows(ra, ag + (size_t)(s - sBegin) * aStage, aPass, SeqA());
         if (PW) ig_load_rows(rv, vg + (size_t)(s - sBegin) * vStage, vPass, SeqBV());
-        else rbOk = ig_gather_rows(rb, ximg, pixOff, maskR, maskS, p.table, s * BK + grow0, TL::ROW_STEP, SeqB());
+        else rbOk = ig_gather_rows<MASKED>(rb, ximg, pixOff, maskR, maskS, p.table, s * BK + grow0, TL::ROW_STEP, SeqB());
     };
     if (sBegin + 1 < sEnd) load_stage(sBegin + 1);
     __syncthreads();
@@ -248,7 +257,7 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
                 // and the one after it is requested at once: a whole stage in flight
                 ig_store_rows(&As[buf ^ 1][aLds], ra, TL::A_ROWS * BM, SeqA());
                 if (PW) ig_store_rows(&Bs[buf ^ 1][vLds], rv, BV_ROWS * BN, SeqBV());
-                else ig_scatter_rows(&Bs[buf ^ 1][bLds], rb, rbOk, TL::ROW_STEP * BN, SeqB());
+                else ig_scatter_rows<MASKED>(&Bs[buf ^ 1][bLds], rb, rbOk, TL::ROW_STEP * BN, SeqB());
                 if (s + 2 < sEnd) load_stage(s + 2);
             }
         }
@@ -385,8 +394,12 @@ void launch(fc_context *ctx, IgemmParams &p) {
     const bool pointwise = p.kh == 1 && p.kw == 1 && p.sh == 1 && p.sw == 1 && p.pt == 0 && p.pl == 0 &&
                            p.OH == p.H && p.OW == p.W && (p.H * p.W) % 4 == 0 && p.C % TL::BK_ == 0 &&
                            ((uintptr_t)p.x & 15) == 0;
-    if (pointwise) igemm_conv_kernel<TL, true><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
-    else igemm_conv_kernel<TL, false><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
+    // no tap of any window leaves the image, and no padding rows in the reduction
+    const bool inside = p.pt == 0 && p.pl == 0 && (p.OH - 1) * p.sh + p.kh <= p.H && (p.OW - 1) * p.sw + p.kw <= p.W &&
+                        (p.C * p.kh * p.kw) % TL::BK_ == 0;
+    if (pointwise) igemm_conv_kernel<TL, IG_POINTWISE><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
+    else if (inside) igemm_conv_kernel<TL, IG_GATHER_INSIDE><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
+    else igemm_conv_kernel<TL, IG_GATHER><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
 }
 
 }  // namespace

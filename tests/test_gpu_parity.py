@@ -241,6 +241,9 @@ IGEMM_SHAPES = [
     # pointwise layers: vector path (pixels per image a multiple of 4) and gather path (7x7 = 49 pixels)
     (32, 64, 56, 56, 256, 1, 1, 1, 1, 0), (3, 70, 6, 6, 33, 1, 1, 1, 1, 0), (5, 20, 7, 7, 40, 1, 1, 1, 1, 0),
     (2, 19, 10, 10, 130, 1, 1, 1, 1, 0),
+    # windows that never leave the image (no padding, whole-stage reduction): the gather without bounds masks
+    (3, 32, 15, 15, 64, 1, 1, 2, 2, 0), (2, 16, 12, 13, 40, 3, 3, 1, 1, 0), (2, 48, 9, 9, 70, 1, 1, 1, 1, 0),
+    (3, 4, 17, 16, 33, 2, 2, 2, 2, 0), (32, 256, 56, 56, 512, 1, 1, 2, 2, 0),
 ]
 
 
