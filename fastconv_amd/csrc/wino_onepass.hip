@@ -386,10 +386,11 @@ extern "C" int fc_wino_prefer_onepass(const fc_conv_shape *s) {
     if (!fc_shape_ok(s) || s->kh != 3 || s->kw != 3 || s->sh != 1 || s->sw != 1 || s->W < 8) return 0;
     if (s->C < 16 || s->C > 64) return 0;
     // one 16-tile x 64-channel block per workgroup, one workgroup per CU at a time: the layer must
-    // bring a few blocks per CU (batch 1 layers do not)
+    // bring a few blocks per CU (batch 1 layers do not).  Measured crossover against the staged
+    // pipeline: about 200 blocks when one block covers all output channels, 500 otherwise.
     const long OH = fc_out_dim(s->H, s->pt, s->pb, 3, 1), OW = fc_out_dim(s->W, s->pl, s->pr, 3, 1);
     const long blocks = ((long)s->N * ((OH + 5) / 6) * ((OW + 5) / 6) + kTB - 1) / kTB * ((s->K + kKB - 1) / kKB);
-    return blocks >= 512 ? 1 : 0;
+    return blocks >= (s->K <= kKB ? 192 : 512) ? 1 : 0;
 }
 
 extern "C" int fc_wino_forward_onepass(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev, const float *w_dev,

@@ -262,7 +262,8 @@ int fc_wino_forward_onepass(fc_context *ctx, const fc_wino_plan *plan, const flo
 /* 1 when the single-kernel path is expected to be the fastest Winograd pipeline for this
  * layer (measured on MI355X: 16 to 64 input channels, where the products are cheap next to
  * moving V and M through HBM, the image at least 8 columns wide, and at least 512 blocks of
- * 16 tiles x 64 output channels, i.e. not at batch 1). */
+ * 16 tiles x 64 output channels -- 192 when one block covers all output channels -- i.e. not
+ * at batch 1). */
 int fc_wino_prefer_onepass(const fc_conv_shape *shape);
 
 /* All stages back to back: what winoF63_v1_single (winoF63ZC/winoF63ZC.h:5-6)
