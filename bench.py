@@ -486,9 +486,18 @@ def main():
         transforms["implicit_gemm"] = {"bound": "mfma", "achieved": round(tf, 2), "peak": PEAK_MFMA_F32_TFLOPS,
                                        "unit": "TFLOP/s", "frac": round(tf / PEAK_MFMA_F32_TFLOPS, 4),
                                        "launches": igemm_stage[1]}
-    if not staged and igemm_stage[1] > 0:      # no staged Winograd layer: the implicit GEMM is the dominant kernel
+    # the dominant kernel is the one with more time in the timed region: the implicit GEMM in the
+    # ResNet-50 workloads, the staged Winograd GEMM in the VGG-16 ones
+    if igemm_stage[1] > 0 and (not staged or igemm_stage[0] > stage[ST_GEMM][0]):
+        wino_gemm_line = roofline if staged and stage[ST_GEMM][1] > 0 else None
         roofline = dict(transforms["implicit_gemm"], kernel="igemm_conv_kernel", traffic=None,
                         avg_launch_ms=round(igemm_stage[0] / igemm_stage[1], 5))
+        if shader_clock:
+            at_clock = info["compute_units"] * 256 * shader_clock["mean_mhz"] * 1e6 / 1e12
+            roofline.update(peak_at_measured_clock=round(at_clock, 1),
+                            frac_at_measured_clock=round(roofline["achieved"] / at_clock, 4))
+        if wino_gemm_line:
+            transforms["wino_gemm"] = wino_gemm_line
 
     # yardstick for the HBM-bound kernels: the library's plain copy kernel (16 bytes per lane) over the
     # V and M scratch, outside the timed region
