@@ -253,13 +253,19 @@ def main():
     ap.add_argument("--offline-filter", action="store_true",
                     help="transform the filters once outside the timed region")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--stage-events", default="gemm", choices=["all", "gemm", "none"],
-                    help="which kernels are bracketed by events inside the timed region (default: the dominant "
-                         "kernel only; an event pair costs about 5 us per launch, so the other kernels are "
-                         "bracketed in a few extra untimed steps after it)")
+    ap.add_argument("--stage-events", default="auto", choices=["auto", "all", "gemm", "none"],
+                    help="which kernels are bracketed by events inside the timed region.  An event pair costs "
+                         "5-8 us per launch: 'gemm' brackets the dominant kernel only (the other kernels are "
+                         "bracketed in a few extra untimed steps), 'none' brackets nothing in the timed region "
+                         "(everything comes from the untimed steps).  'auto' (default) is 'gemm' when a step "
+                         "holds at most 16 such launches (the VGG-16 workloads: 9-13), else 'none' (ResNet-50: "
+                         "53 launches, where the brackets would add 15 %% to the step)")
     ap.add_argument("--pipeline", default="auto", choices=["auto", "staged", "fused", "onepass"],
                     help="Winograd pipeline per layer: four staged kernels, GEMM + output transform fused, or "
                          "whichever is faster for the layer (auto)")
+    ap.add_argument("--graph", action="store_true",
+                    help="record one step as a HIP graph and time replays of it (per-launch events are off; "
+                         "the default times the per-layer calls the reference's driver makes)")
     ap.add_argument("--timed-only", action="store_true",
                     help="no per-layer detail pass after the timed region (every launch of the process is then a "
                          "warm-up or timed step: what a kernel trace of this command averages over)")
@@ -355,12 +361,24 @@ def main():
         step()
     L.sync()
 
+    if args.stage_events == "auto":
+        bracketed = sum(l.repeats for l in layers if l.algo == "im2col" or l.pipe == "staged")
+        args.stage_events = "gemm" if bracketed <= 16 else "none"
     mask = {"all": 0xdf, "gemm": (1 << ST_GEMM) | (1 << 4), "none": 0}[args.stage_events]
+    timed_step = step
+    if args.graph:
+        mask = 0
+        L.graph_begin()
+        step()
+        recorded = L.graph_end()
+        timed_step = lambda: L.graph_launch(recorded)
+        timed_step()
+        L.sync()
     L.timing(mask)
     L.timing_reset()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step()
+        timed_step()
     L.sync()
     elapsed = time.perf_counter() - t0
     stage = [L.stage_time(i) for i in range(4)]
@@ -380,7 +398,7 @@ def main():
             stage[i] = detail[i]
         fused_stage = L.stage_time(6)
         onepass_stage = L.stage_time(7)
-        if args.stage_events == "none":
+        if args.stage_events == "none" or args.graph:
             stage[ST_GEMM] = detail[ST_GEMM]
             igemm_stage = L.stage_time(4)
         L.timing(0)
@@ -555,6 +573,8 @@ def main():
         per_layer.append(row)
     L.timing(0)
 
+    roofline["events"] = ("inside the timed region" if args.stage_events in ("gemm", "all") and not args.graph
+                          else "in the untimed steps after it")
     out = {
         "metric": "effective GFLOP/s over the conv stack (direct-conv FLOP count / time)",
         "value": round(value, 1), "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -564,7 +584,8 @@ def main():
                    "per_layer": ",".join("im2col" if l.algo == "im2col" else "wino-" + l.pipe
                                          for l in layers),
                    "filter_transform": "offline" if filter_ready else "online (inside the timed region)",
-                   "tuned": not args.no_tune, "stage_events": args.stage_events,
+                   "tuned": not args.no_tune, "stage_events": "none" if args.graph else args.stage_events,
+                   "launch": "hip graph replay" if args.graph else "per-layer calls",
                    "device": info["arch"], "compute_units": info["compute_units"], "clock_mhz": info["clock_mhz"]},
         "roofline": roofline,
         "shader_clock": shader_clock,
