@@ -257,9 +257,9 @@ def main():
                     help="which kernels are bracketed by events inside the timed region.  An event pair costs "
                          "5-8 us per launch: 'gemm' brackets the dominant kernel only (the other kernels are "
                          "bracketed in a few extra untimed steps), 'none' brackets nothing in the timed region "
-                         "(everything comes from the untimed steps).  'auto' (default) is 'gemm' when a step "
-                         "holds at most 16 such launches (the VGG-16 workloads: 9-13), else 'none' (ResNet-50: "
-                         "53 launches, where the brackets would add 15 %% to the step)")
+                         "(everything comes from the untimed steps).  'auto' (default) is 'gemm' while the "
+                         "brackets cost under 2 %% of a step (VGG-16 at batch 32: 9 launches in 3.5 ms), else "
+                         "'none' (ResNet-50: 53 launches, 15 %% of the step; batch-1 stacks)")
     ap.add_argument("--pipeline", default="auto", choices=["auto", "staged", "fused", "onepass"],
                     help="Winograd pipeline per layer: four staged kernels, GEMM + output transform fused, or "
                          "whichever is faster for the layer (auto)")
@@ -362,8 +362,14 @@ def main():
     L.sync()
 
     if args.stage_events == "auto":
+        # one more untimed step for a rough step time: brackets stay inside the timed region while
+        # their own cost (about 6 us per bracketed launch) is under 2 % of the step
+        t0 = time.perf_counter()
+        step()
+        L.sync()
+        rough_us = (time.perf_counter() - t0) * 1e6
         bracketed = sum(l.repeats for l in layers if l.algo == "im2col" or l.pipe == "staged")
-        args.stage_events = "gemm" if bracketed <= 16 else "none"
+        args.stage_events = "gemm" if 6.0 * bracketed <= 0.02 * rough_us else "none"
     mask = {"all": 0xdf, "gemm": (1 << ST_GEMM) | (1 << 4), "none": 0}[args.stage_events]
     timed_step = step
     if args.graph:
