@@ -200,6 +200,39 @@ def test_pipelines_agree_on_random_shapes(lib):
             assert O.max_rel_err(y, truth) <= TOL_WINO, name
 
 
+def test_implicit_gemm_on_random_geometries(lib):
+    """60 seeded random convolutions (filter 1..5, stride 1..3, asymmetric padding 0..2, channel
+    counts around the tile sizes, random tile shape) against the fp64 oracle: whichever of the
+    pointwise, unmasked-gather and masked-gather kernels and of the two epilogues a geometry selects."""
+    rng = np.random.default_rng(4321)
+    ncfg = len(lib.igemm_configs())
+    done = 0
+    for case in range(80):
+        N, C = int(rng.integers(1, 4)), int(rng.choice([1, 3, 8, 16, 20, 32, 48, 64]))
+        K = int(rng.choice([1, 7, 32, 64, 72, 128, 256]))
+        kh, kw = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        sh, sw = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        H, W = int(rng.integers(4, 24)), int(rng.integers(4, 24))
+        pt, pb, pl, pr = (int(v) for v in rng.integers(0, 3, size=4))
+        if H + pt + pb < kh or W + pl + pr < kw:
+            continue
+        geo = (N, C, H, W, K, kh, kw, sh, sw, pt, pb, pl, pr)
+        s = O.Shape(*geo)
+        cfg = int(rng.integers(0, ncfg))
+        x, w = O.make_inputs(s, seed=100 + case)
+        use_bias, relu = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        bias = O.rng_uniform(case, (K,)) if use_bias else None
+        announce("random geometry", case, geo, "tile config", cfg, "bias", use_bias, "relu", relu)
+        truth = O.naive_conv_f64(s, x, w, bias)
+        if relu:
+            truth = np.maximum(truth, 0.0)
+        y = lib.implicit_gemm_conv(cshape(s), x, w, bias=bias, relu=relu, config=cfg)
+        assert y.shape == truth.shape
+        assert O.max_rel_err(y, truth) <= TOL_IM2COL, (case, geo, cfg)
+        done += 1
+    assert done >= 60
+
+
 def test_winograd_single_kernel_refuses_narrow_images(lib):
     import fastconv_amd as F
     with pytest.raises(F.FastConvError) as e:
