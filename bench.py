@@ -66,6 +66,7 @@ WORKLOADS = {
     "resnet50_3x3_b1": (_w(RESNET50_3X3), 1, "winograd", "ResNet-50 3x3 s1 convs, Winograd F(6,3), batch 1"),
     "im2col_abc_b1": (IM2COL_ABC, 1, "im2col", "BASELINE config 2: 3x3 256@56, 3x3 s2 128->256@56, 1x1 256->1024@14, batch 1"),
     "cfg1": (_w([(64, 64, 56, 1)]), 1, "winograd", "single 3x3 conv 64->64 @56, batch 1"),
+    "conv64_224_b32": (_w([(64, 64, 224, 1)]), 32, "winograd", "single 3x3 conv 64->64 @224, batch 32 (VGG-16 layer 2)"),
     "stress_b64": (_w(STRESS), 64, "winograd", "VGG-16 256@56, 512@28, 512@14, batch 64"),
     "stress_b128": (_w(STRESS), 128, "winograd", "VGG-16 256@56, 512@28, 512@14, batch 128"),
 }
