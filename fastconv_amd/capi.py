@@ -9,7 +9,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libfastconv_hip.so")
 
 STAGE_NAMES = ["KernelTran", "InputTran", "TensorGEMM", "OutputTran", "ImplicitGemm", "FilterPack",
-               "FusedGemmOut"]
+               "FusedGemmOut", "OnePass"]
 
 
 class FastConvError(RuntimeError):
@@ -90,6 +90,7 @@ _ABI = {
     "fc_wino_gemm_get_config": (C.c_int, [C.c_int, C.POINTER(GemmConfig)]),
     "fc_wino_gemm_default_config": (C.c_int, [C.POINTER(ConvShape)]),
     "fc_igemm_default_config": (C.c_int, [C.POINTER(ConvShape)]),
+    "fc_prefer_winograd": (C.c_int, [C.POINTER(ConvShape)]),
     "fc_wino_make_plan": (C.c_int, [C.POINTER(ConvShape), C.c_int, C.POINTER(WinoPlan)]),
     "fc_wino_filter_transform": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp]),
     "fc_wino_input_transform": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp]),
@@ -190,15 +191,23 @@ class Library:
         self._check(self.c.fc_pool_stats(self.pool, C.byref(a), C.byref(b), C.byref(c_)))
         return a.value, b.value, c_.value
 
+    @staticmethod
+    def _host_array(arr):
+        """Host data as the kernels read it: C-contiguous float32 (int32 arrays pass unchanged)."""
+        arr = np.asarray(arr)
+        if arr.dtype != np.int32:
+            arr = arr.astype(np.float32, copy=False)
+        return np.ascontiguousarray(arr)
+
     def upload(self, arr):
-        arr = np.ascontiguousarray(arr)
+        arr = self._host_array(arr)
         p = self.alloc(max(arr.nbytes, 4))
         self._check(self.c.fc_upload(self.ctx, p, arr.ctypes.data_as(_vp), arr.nbytes))
         return p
 
     def upload_into(self, ptr, arr):
         """Copy a host array into device memory that was allocated before."""
-        arr = np.ascontiguousarray(arr)
+        arr = self._host_array(arr)
         self._check(self.c.fc_upload(self.ctx, ptr, arr.ctypes.data_as(_vp), arr.nbytes))
 
     def download(self, ptr, shape, dtype=np.float32):
@@ -290,6 +299,10 @@ class Library:
 
     def igemm_default_config(self, shape):
         return self.c.fc_igemm_default_config(C.byref(shape))
+
+    def prefer_winograd(self, shape):
+        """The library's rule behind `-a auto` for this layer."""
+        return bool(self.c.fc_prefer_winograd(C.byref(shape)))
 
     def wino_plan(self, shape, config=0):
         plan = WinoPlan()

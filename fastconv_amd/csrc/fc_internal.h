@@ -88,6 +88,26 @@ static inline bool fc_shape_ok(const fc_conv_shape *s) {
     return true;
 }
 
+static inline bool fc_same_shape(const fc_conv_shape &a, const fc_conv_shape &b) {
+    return a.N == b.N && a.C == b.C && a.H == b.H && a.W == b.W && a.K == b.K && a.kh == b.kh && a.kw == b.kw &&
+           a.sh == b.sh && a.sw == b.sw && a.pt == b.pt && a.pb == b.pb && a.pl == b.pl && a.pr == b.pr;
+}
+
+// Every field of a plan a caller hands in is compared with the plan the library itself makes
+// for the same shape and configuration: the kernels take their sizes from it unverified.
+static inline bool fc_same_wino_plan(const fc_wino_plan &a, const fc_wino_plan &b) {
+    return fc_same_shape(a.shape, b.shape) && a.OH == b.OH && a.OW == b.OW && a.tiles_h == b.tiles_h &&
+           a.tiles_w == b.tiles_w && a.T == b.T && a.K_pad == b.K_pad && a.C_pad == b.C_pad && a.T_pad == b.T_pad &&
+           a.gemm_config == b.gemm_config && a.U_bytes == b.U_bytes && a.V_bytes == b.V_bytes && a.M_bytes == b.M_bytes;
+}
+
+static inline bool fc_same_igemm_plan(const fc_igemm_plan &a, const fc_igemm_plan &b) {
+    return fc_same_shape(a.shape, b.shape) && a.OH == b.OH && a.OW == b.OW && a.Kred == b.Kred &&
+           a.Kred_pad == b.Kred_pad && a.K_pad == b.K_pad && a.Npix == b.Npix && a.config == b.config &&
+           a.Wp_bytes == b.Wp_bytes && a.table_bytes == b.table_bytes && a.split_k == b.split_k &&
+           a.ws_bytes == b.ws_bytes;
+}
+
 // Unsigned division by a runtime constant: q = (n * mul) >> (32 + shift), exact
 // for n < 2^31 (round-up method with a 33-bit multiplier folded by one add).
 struct fc_fastdiv {

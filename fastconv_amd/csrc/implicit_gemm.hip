@@ -486,8 +486,7 @@ static int ig_plan_check(fc_context *ctx, const fc_igemm_plan *plan) {
     fc_igemm_plan chk;
     const int rc = fc_igemm_make_plan(&plan->shape, plan->config, &chk);
     if (rc) return fc_set_error(ctx, rc, "plan does not describe a supported layer", hipSuccess);
-    if (chk.Kred_pad != plan->Kred_pad || chk.K_pad != plan->K_pad || chk.Npix != plan->Npix ||
-        chk.split_k != plan->split_k || chk.ws_bytes != plan->ws_bytes)
+    if (!fc_same_igemm_plan(chk, *plan))
         return fc_set_error(ctx, FC_ERR_INVALID, "plan fields were modified after fc_igemm_make_plan", hipSuccess);
     return FC_OK;
 }

@@ -111,8 +111,7 @@ extern "C" int fc_wino_gemm_output_fused(fc_context *ctx, const fc_wino_plan *pl
     if (!plan || !U_dev || !V_dev || !y_dev)
         return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_gemm_output_fused: null argument", hipSuccess);
     fc_wino_plan chk;
-    if (fc_wino_make_plan(&plan->shape, plan->gemm_config, &chk) != FC_OK || chk.K_pad != plan->K_pad ||
-        chk.C_pad != plan->C_pad || chk.T_pad != plan->T_pad || chk.T != plan->T)
+    if (fc_wino_make_plan(&plan->shape, plan->gemm_config, &chk) != FC_OK || !fc_same_wino_plan(chk, *plan))
         return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_gemm_output_fused: plan does not describe a supported layer", hipSuccess);
     if ((size_t)plan->C_pad * plan->T_pad >= (1ull << 30) || (size_t)plan->C_pad * plan->K_pad >= (1ull << 30))
         return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_gemm_output_fused: a frequency plane of U or V exceeds 4 GiB", hipSuccess);

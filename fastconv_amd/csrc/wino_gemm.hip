@@ -331,6 +331,9 @@ extern "C" int fc_wino_gemm(fc_context *ctx, const fc_wino_plan *plan, const flo
     if (!plan || !U_dev || !V_dev || !M_dev) return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_gemm: null argument", hipSuccess);
     fc_gemm_config cfg;
     if (fc_wino_gemm_get_config(plan->gemm_config, &cfg)) return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_gemm: unknown tile configuration", hipSuccess);
+    fc_wino_plan chk;
+    if (fc_wino_make_plan(&plan->shape, plan->gemm_config, &chk) != FC_OK || !fc_same_wino_plan(chk, *plan))
+        return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_gemm: plan fields were modified after fc_wino_make_plan", hipSuccess);
     // the kernel has no edge predication: the buffers must be padded to the tile
     if (plan->K_pad <= 0 || plan->C_pad <= 0 || plan->T_pad <= 0 || plan->K_pad % cfg.bm || plan->C_pad % cfg.bk ||
         plan->T_pad % cfg.bn)

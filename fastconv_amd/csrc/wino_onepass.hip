@@ -310,8 +310,7 @@ int onepass_plan_check(fc_context *ctx, const fc_wino_plan *plan, const void *a,
     fc_wino_plan chk;
     const int rc = fc_wino_make_onepass_plan(&plan->shape, &chk);
     if (rc) return fc_set_error(ctx, rc, "plan does not describe a layer the single-kernel path supports", hipSuccess);
-    if (plan->gemm_config != FC_WINO_ONEPASS || chk.K_pad != plan->K_pad || chk.C_pad != plan->C_pad ||
-        chk.T_pad != plan->T_pad || chk.T != plan->T)
+    if (plan->gemm_config != FC_WINO_ONEPASS || !fc_same_wino_plan(chk, *plan))
         return fc_set_error(ctx, FC_ERR_INVALID, "not a plan made by fc_wino_make_onepass_plan", hipSuccess);
     return FC_OK;
 }

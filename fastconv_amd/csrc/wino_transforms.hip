@@ -287,6 +287,8 @@ __global__ __launch_bounds__(TPB) void wino_output_transform_kernel(const OutTPa
     }
 }
 
+constexpr int kWinoMaxTilesW = 170;
+
 // Largest of 128 / 64 / 32 tiles per block that divides the padded tile count.
 int tiles_per_block(long T_pad) { return (T_pad % 128 == 0) ? 128 : (T_pad % 64 == 0) ? 64 : 32; }
 
@@ -313,11 +315,25 @@ extern "C" int fc_wino_make_plan(const fc_conv_shape *s, int gemm_config, fc_win
     plan->U_bytes = sizeof(float) * 64 * (size_t)plan->C_pad * plan->K_pad;
     plan->V_bytes = sizeof(float) * 64 * (size_t)plan->C_pad * plan->T_pad;
     plan->M_bytes = sizeof(float) * 64 * (size_t)plan->K_pad * plan->T_pad;
-    if (plan->tiles_w > 256) return FC_ERR_UNSUPPORTED;       // output wider than 1536
+    // output wider than 1020: a band of the input transform (8 rows x 6*tiles_w + 2 columns, two of them
+    // per workgroup) no longer fits 64 KiB of LDS
+    if (plan->tiles_w > kWinoMaxTilesW) return FC_ERR_UNSUPPORTED;
     if (plan->T_pad >= (1l << 31) || (size_t)plan->C_pad * plan->T_pad >= (1ull << 31) ||
         (size_t)plan->K_pad * plan->T_pad >= (1ull << 31))
         return FC_ERR_UNSUPPORTED;
     return FC_OK;
+}
+
+extern "C" int fc_prefer_winograd(const fc_conv_shape *s) {
+    if (!fc_shape_ok(s) || s->kh != 3 || s->kw != 3 || s->sh != 1 || s->sw != 1) return 0;
+    const int OH = fc_out_dim(s->H, s->pt, s->pb, 3, 1), OW = fc_out_dim(s->W, s->pl, s->pr, 3, 1);
+    const long tilesW = (OW + 5) / 6, tiles = (long)s->N * ((OH + 5) / 6) * tilesW;
+    if (tilesW > kWinoMaxTilesW) return 0;
+    // few input channels: the M planes (64 floats per 36 outputs) dominate and carry no reuse
+    if (s->C < 16) return 0;
+    // few tiles: the 64x larger transformed filter dominates
+    if (tiles < 64 && (long)s->C * s->K >= 128 * 128) return 0;
+    return 1;
 }
 
 static int plan_check(fc_context *ctx, const fc_wino_plan *plan, const void *a, const void *b) {
@@ -326,7 +342,7 @@ static int plan_check(fc_context *ctx, const fc_wino_plan *plan, const void *a, 
     fc_wino_plan chk;
     const int rc = fc_wino_make_plan(&plan->shape, plan->gemm_config, &chk);
     if (rc) return fc_set_error(ctx, rc, "plan does not describe a supported layer", hipSuccess);
-    if (chk.K_pad != plan->K_pad || chk.C_pad != plan->C_pad || chk.T_pad != plan->T_pad || chk.T != plan->T)
+    if (!fc_same_wino_plan(chk, *plan))
         return fc_set_error(ctx, FC_ERR_INVALID, "plan fields were modified after fc_wino_make_plan", hipSuccess);
     return FC_OK;
 }
@@ -363,16 +379,22 @@ static int launch_input_transform(fc_context *ctx, const fc_wino_plan *plan, con
     p.divLW = fc_make_fastdiv(p.LW);
     p.divTH = fc_make_fastdiv(p.tH);
     p.divTW = fc_make_fastdiv(p.tW);
-    const int tpb = tiles_per_block(plan->T_pad);
-    // a range of tpb tiles touches at most this many bands
-    const int maxBands = (tpb + p.tW - 2) / p.tW + 1;
-    const size_t ldsBytes = (size_t)maxBands * 8 * p.LW * sizeof(float);
+    // The largest of 128 / 64 / 32 tiles per block that divides the padded tile count and whose bands
+    // fit 64 KiB of LDS (a range of tpb tiles touches at most maxBands bands of 8 rows x LW columns).
+    // fc_wino_make_plan admits at most 170 tiles per band, for which 32 tiles per block always fit.
+    int tpb = tiles_per_block(plan->T_pad), maxBands = 0;
+    size_t ldsBytes = 0;
+    for (;; tpb /= 2) {
+        maxBands = (tpb + p.tW - 2) / p.tW + 1;
+        ldsBytes = (size_t)maxBands * 8 * p.LW * sizeof(float);
+        if (ldsBytes <= 64 * 1024 || tpb == 32) break;
+    }
     if (ldsBytes > 64 * 1024) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_input_transform: image too wide", hipSuccess);
     const dim3 grid((unsigned)(plan->T_pad / tpb), plan->C_pad);
     if (grid.y > 65535) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_input_transform: more than 65535 channels", hipSuccess);
-    // columns (band x column pairs) per thread in pass 1
+    // columns (band x column pairs) per thread in pass 1: at most 8, since maxBands * LW <= 2048
     const int itemsPerThread = (maxBands * p.LW + 255) / 256;
-    if (itemsPerThread > 6) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_input_transform: image too wide", hipSuccess);
+    if (itemsPerThread > 8) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_input_transform: image too wide", hipSuccess);
     const int filterGridX = (plan->K_pad + 63) / 64;
     const long nFilter = q ? (long)filterGridX * ((plan->C_pad + 3) / 4) : 0;
     const long total = nFilter + (long)grid.x * grid.y;
@@ -390,7 +412,8 @@ static int launch_input_transform(fc_context *ctx, const fc_wino_plan *plan, con
     do {                                                     \
         if (itemsPerThread <= 2) FC_LAUNCH_ONE(TPB_, 2);     \
         else if (itemsPerThread <= 4) FC_LAUNCH_ONE(TPB_, 4); \
-        else FC_LAUNCH_ONE(TPB_, 6);                         \
+        else if (itemsPerThread <= 6) FC_LAUNCH_ONE(TPB_, 6); \
+        else FC_LAUNCH_ONE(TPB_, 8);                         \
     } while (0)
     if (tpb == 128) FC_LAUNCH_INT(128);
     else if (tpb == 64) FC_LAUNCH_INT(64);
@@ -430,9 +453,14 @@ extern "C" int fc_wino_output_transform(fc_context *ctx, const fc_wino_plan *pla
     p.T = plan->T; p.K_pad = plan->K_pad; p.T_pad = plan->T_pad;
     p.divTH = fc_make_fastdiv(p.tH);
     p.divTW = fc_make_fastdiv(p.tW);
-    const int tpb = (plan->T_pad % 128 == 0 && plan->T >= 128) ? 128 : 64;
-    const int maxBands = (tpb + p.tW - 2) / p.tW + 1;
-    const size_t ldsBytes = (size_t)maxBands * 6 * p.OW * sizeof(float);
+    int tpb = (plan->T_pad % 128 == 0 && plan->T >= 128) ? 128 : 64;
+    int maxBands = (tpb + p.tW - 2) / p.tW + 1;
+    size_t ldsBytes = (size_t)maxBands * 6 * p.OW * sizeof(float);
+    if (ldsBytes > 64 * 1024 && tpb == 128) {
+        tpb = 64;
+        maxBands = (tpb + p.tW - 2) / p.tW + 1;
+        ldsBytes = (size_t)maxBands * 6 * p.OW * sizeof(float);
+    }
     if (ldsBytes > 64 * 1024) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_output_transform: image too wide", hipSuccess);
     const dim3 grid((unsigned)((plan->T + tpb - 1) / tpb), s.K);
     if (grid.y > 65535) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_output_transform: more than 65535 channels", hipSuccess);

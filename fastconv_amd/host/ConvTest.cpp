@@ -49,6 +49,7 @@ struct options {
     bool blocked_variant;
     bool variant_given;
     bool check;
+    size_t check_images;
     bool strict;
     bool json;
 };
@@ -74,6 +75,8 @@ void print_options_help(const char *program_name) {
         "       --variant            Winograd pipeline: zc (four staged kernels) or blocked (no M buffer / single kernel);\n"
         "                            default: whichever the library prefers for the layer\n"
         "       --no-check           Skip the naive reference and the error check\n"
+        "       --check-images       Check only the last K images of the batch against the naive reference\n"
+        "                            (default: all; the host convolution of a large batch takes minutes)\n"
         "       --strict             Exit with status 2 when the error exceeds the tolerance\n"
         "       --json               Also print one JSON line with the results\n",
         program_name);
@@ -129,6 +132,7 @@ struct options parse_options(int argc, char **argv) {
     options.blocked_variant = false;
     options.variant_given = false;
     options.check = true;
+    options.check_images = 0;
     options.strict = false;
     options.json = false;
 
@@ -211,6 +215,9 @@ struct options parse_options(int argc, char **argv) {
             i += 1;
         } else if (is_flag(argv[i], "--no-check", NULL)) {
             options.check = false;
+        } else if (is_flag(argv[i], "--check-images", NULL)) {
+            options.check_images = parse_count(argc, argv, i, "number of checked images", false);
+            i += 1;
         } else if (is_flag(argv[i], "--strict", NULL)) {
             options.strict = true;
         } else if (is_flag(argv[i], "--json", NULL)) {
@@ -294,21 +301,30 @@ int main(int argc, char *argv[]) {
     fillTestInput(test_input, options.batch, (int)input_channels, input_size, options.seed);
     fillTestKernel(test_kernel, (int)input_channels, (int)output_channels, kernel_size, options.seed);
 
+    // the naive reference covers the whole batch, or its last --check-images images
+    const size_t checked = (options.check_images && options.check_images < options.batch) ? options.check_images : options.batch;
+    const size_t first_checked = options.batch - checked;
+    const bool partial_check = checked < options.batch;
     ConvNaiveLayer *conv_reference = NULL;
     double naive_ms = 0.0;
     if (options.check) {
-        conv_reference = new ConvNaiveLayer(test_input, test_kernel, NULL, NULL, input_channels, input_size.height,
+        conv_reference = new ConvNaiveLayer(test_input + first_checked * (in_elems / options.batch), test_kernel, NULL, NULL,
+                                            input_channels, input_size.height,
                                             input_size.width, output_channels, kernel_size.height, kernel_size.width,
                                             output_subsampling.height, output_subsampling.width, input_padding.left,
                                             input_padding.right, input_padding.top, input_padding.bottom, 1, false,
-                                            options.threads, 1, options.batch);
+                                            options.threads, 1, checked);
         Timer naive;
         naive.startBench();
         conv_reference->Forward();
         naive_ms = naive.endBench(1.0);
-        printf("Naive reference on %zu host thread(s): %.3f ms\n", options.threads, naive_ms);
+        printf("Naive reference on %zu host thread(s), %zu of %zu image(s): %.3f ms\n", options.threads, checked,
+               options.batch, naive_ms);
     }
     float *output_ref = conv_reference ? conv_reference->output_data : NULL;
+    // the layers compare their whole output with the array they are given (the reference's diff()):
+    // with a partial reference that comparison is made here instead
+    float *layer_ref = partial_check ? NULL : output_ref;
 
     if (options.algorithm == nnp_convolution_algorithm_auto)
         options.algorithm = select_algorithm(kernel_size, output_subsampling, output_size, input_channels,
@@ -338,6 +354,8 @@ int main(int argc, char *argv[]) {
     ConvLayer *conv_test = NULL;
     double tolerance = 1e-5;
     int chosen_config = -1;
+    int chosen_option = -1;                 // blocked Winograd: images per block (0 = single-kernel engine)
+    int kernel_transform_offline = -1;      // Winograd: 1 = filter transformed once in Init(), 0 = in every pass
     double stage_ms[4] = {0, 0, 0, 0};
     switch (options.algorithm) {
         case nnp_convolution_algorithm_auto:
@@ -346,7 +364,7 @@ int main(int argc, char *argv[]) {
         case nnp_convolution_algorithm_im2col: {
             // "direct" (1x1 stride 1) is the same kernel: with a 1x1 window the gather is a plain row read
             ConvIm2colLayer *conv = new ConvIm2colLayer(
-                test_input, test_kernel, NULL, output_ref, input_channels, input_size.height, input_size.width,
+                test_input, test_kernel, NULL, layer_ref, input_channels, input_size.height, input_size.width,
                 output_channels, kernel_size.height, kernel_size.width, output_subsampling.height,
                 output_subsampling.width, input_padding.left, input_padding.right, input_padding.top,
                 input_padding.bottom, 1, false, options.threads, options.iterations, options.batch);
@@ -368,19 +386,22 @@ int main(int argc, char *argv[]) {
             }
             if (options.blocked_variant) {
                 ConvWinoF63Layer *conv = new ConvWinoF63Layer(
-                    test_input, test_kernel, NULL, output_ref, input_channels, input_size.height, input_size.width,
+                    test_input, test_kernel, NULL, layer_ref, input_channels, input_size.height, input_size.width,
                     output_channels, kernel_size.height, kernel_size.width, output_subsampling.height,
                     output_subsampling.width, input_padding.left, input_padding.right, input_padding.top,
                     input_padding.bottom, 1, false, options.threads, options.iterations, options.batch);
                 if (options.tuning_strategy != nnp_convolution_tuning_strategy_no_tuning) conv->Tuning();
+                else conv->SetOfflineKernelTransform(options.transform_strategy == nnp_convolution_transform_strategy_offline);
                 conv->Init();
                 conv->Forward();
                 chosen_config = conv->best_config();
+                chosen_option = conv->best_images_per_block();
+                kernel_transform_offline = conv->best_offline();
                 for (int i = 0; i < 4; i++) stage_ms[i] = conv->stage_ms[i];
                 conv_test = conv;
             } else {
                 ConvWinoF63ZCLayer *conv = new ConvWinoF63ZCLayer(
-                    test_input, test_kernel, NULL, output_ref, input_channels, input_size.height, input_size.width,
+                    test_input, test_kernel, NULL, layer_ref, input_channels, input_size.height, input_size.width,
                     output_channels, kernel_size.height, kernel_size.width, output_subsampling.height,
                     output_subsampling.width, input_padding.left, input_padding.right, input_padding.top,
                     input_padding.bottom, 1, false, options.threads, options.iterations, options.batch);
@@ -391,6 +412,7 @@ int main(int argc, char *argv[]) {
                 conv->Init();
                 conv->Forward();
                 chosen_config = conv->best_config();
+                kernel_transform_offline = conv->best_offline();
                 for (int i = 0; i < 4; i++) stage_ms[i] = conv->stage_ms[i];
                 conv_test = conv;
             }
@@ -405,7 +427,8 @@ int main(int argc, char *argv[]) {
                conv_test->flops() / 1e9, ms);
         double err = -1.0;
         if (output_ref) {
-            err = max_rel_err(conv_test->output_data, output_ref, out_elems);
+            const size_t out_img = out_elems / options.batch;
+            err = max_rel_err(conv_test->output_data + first_checked * out_img, output_ref, checked * out_img);
             const bool ok = err <= tolerance;
             printf("Max relative error vs naive: %.3e (tolerance %.0e) %s\n", err, tolerance, ok ? "PASS" : "FAIL");
             if (!ok && options.strict) status = 2;
@@ -414,13 +437,15 @@ int main(int argc, char *argv[]) {
             printf("{\"algorithm\": \"%s%s\", \"batch\": %zu, \"ic\": %zu, \"oc\": %zu, \"ih\": %zu, \"iw\": %zu, "
                    "\"kh\": %zu, \"kw\": %zu, \"stride\": %zu, \"pad\": %zu, \"config\": %d, \"ms\": %.6f, "
                    "\"gflops\": %.2f, \"input_tran_ms\": %.6f, \"kernel_tran_ms\": %.6f, \"gemm_ms\": %.6f, "
-                   "\"output_tran_ms\": %.6f, \"max_rel_err\": %.4e, \"naive_ms\": %.3f, \"naive_threads\": %zu}\n",
+                   "\"output_tran_ms\": %.6f, \"max_rel_err\": %.4e, \"naive_ms\": %.3f, \"naive_threads\": %zu, "
+                   "\"checked_images\": %zu, \"images_per_block\": %d, \"kernel_transform\": \"%s\"}\n",
                    algorithm_name(options.algorithm),
                    (options.algorithm == nnp_convolution_algorithm_winograd && options.blocked_variant) ? "_blocked" : "",
                    options.batch, input_channels, output_channels, input_size.height, input_size.width,
                    kernel_size.height, kernel_size.width, output_subsampling.height, options.input_padding,
                    chosen_config, ms, gflops, stage_ms[0], stage_ms[1], stage_ms[2], stage_ms[3], err, naive_ms,
-                   options.threads);
+                   options.threads, options.check ? checked : (size_t)0, chosen_option,
+                   kernel_transform_offline < 0 ? "n/a" : kernel_transform_offline ? "offline" : "online");
         }
     }
     delete conv_test;

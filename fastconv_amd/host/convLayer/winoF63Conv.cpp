@@ -28,7 +28,7 @@ ConvWinoF63Layer::ConvWinoF63Layer(float *input, float *kernel, float *biasw, fl
     gemmConfig_best = ConvWinoF63ZCLayer::DefaultConfig(oc, ic, ih, iw, pad_top, imgBlock_best);
     const fc_conv_shape whole = Shape((int)n);
     if (fc_wino_prefer_onepass(&whole)) imgBlock_best = 0;      // 0: the single-kernel engine, whole batch
-    enableOffKernel = 1;
+    enableOffKernel = enableOffKernel_best = 0;      // online, as the driver's -ts default
     tileBlock = ocBlock = icBlock = ocRegBlock = tileRegBlock = imgBlock = 0;
 }
 
@@ -79,7 +79,8 @@ void ConvWinoF63Layer::AllocateFor(int config, int images_per_block) {
         tileBlock = 16;
         inputBuf = gemmBuf = NULL;
         kernelBuf = (float *)d.Alloc(plan.U_bytes, "kernelBuf");
-        d.Check(fc_wino_onepass_filter_transform(d.ctx(), &plan, dev.kernel, kernelBuf), "fc_wino_onepass_filter_transform");
+        if (enableOffKernel)
+            d.Check(fc_wino_onepass_filter_transform(d.ctx(), &plan, dev.kernel, kernelBuf), "fc_wino_onepass_filter_transform");
         return;
     }
     imgBlock = images_per_block;
@@ -103,22 +104,29 @@ void ConvWinoF63Layer::AllocateFor(int config, int images_per_block) {
     gemmBuf = NULL;      // the per-frequency products live in registers and LDS only
     kernelBuf = (float *)d.Alloc(plan.U_bytes, "kernelBuf");
     // U does not depend on the batch: one transform serves the full and the tail plan
-    d.Check(fc_wino_filter_transform(d.ctx(), &plan, dev.kernel, kernelBuf), "fc_wino_filter_transform");
+    if (enableOffKernel)
+        d.Check(fc_wino_filter_transform(d.ctx(), &plan, dev.kernel, kernelBuf), "fc_wino_filter_transform");
 }
 
-void ConvWinoF63Layer::RunOnce() {
+// split_stages: an online filter transform gets a launch of its own (otherwise it rides in the input
+// transform's launch), so that its time can be listed by itself.
+void ConvWinoF63Layer::RunOnce(bool split_stages) {
     Device &d = Device::Get();
     const size_t in_img = input_channels * input_height * input_width;
     const size_t out_img = output_channels * output_height * output_width;
     if (onePass) {
-        d.Check(fc_wino_conv_onepass(d.ctx(), &plan, dev.input, kernelBuf, dev.bias, relu ? 1 : 0, dev.output),
-                "fc_wino_conv_onepass");
+        d.Check(fc_wino_forward_onepass(d.ctx(), &plan, dev.input, dev.kernel, dev.bias, relu ? 1 : 0, enableOffKernel,
+                                        kernelBuf, dev.output),
+                "fc_wino_forward_onepass");
         return;
     }
+    const bool split = split_stages && !enableOffKernel;
+    if (split) d.Check(fc_wino_filter_transform(d.ctx(), &plan, dev.kernel, kernelBuf), "fc_wino_filter_transform");
     for (size_t n0 = 0; n0 < batch; n0 += imgBlock) {
         const fc_wino_plan *p = (n0 + imgBlock <= batch) ? &plan : &tailPlan;
-        d.Check(fc_wino_forward_fused(d.ctx(), p, dev.input + n0 * in_img, dev.kernel, dev.bias, relu ? 1 : 0, 1,
-                                      kernelBuf, inputBuf, dev.output + n0 * out_img),
+        // online: the filter is transformed with the first block of every pass
+        d.Check(fc_wino_forward_fused(d.ctx(), p, dev.input + n0 * in_img, dev.kernel, dev.bias, relu ? 1 : 0,
+                                      (enableOffKernel || split || n0 > 0) ? 1 : 0, kernelBuf, inputBuf, dev.output + n0 * out_img),
                 "fc_wino_forward_fused");
     }
 }
@@ -126,13 +134,15 @@ void ConvWinoF63Layer::RunOnce() {
 int ConvWinoF63Layer::Tuning() {
     Device &d = Device::Get();
     const fc_conv_shape s = Shape((int)batch);
-    TuningKey key = {"winograd", s.N, s.C, s.H, s.W, s.K, 3, 3, 1, 1, s.pt, s.pb, s.pl, s.pr};
+    TuningKey key = {"winograd_blocked", s.N, s.C, s.H, s.W, s.K, 3, 3, 1, 1, s.pt, s.pb, s.pl, s.pr};
     TuningEntry hit;
     if (tuning_log_lookup(key, &hit) && hit.config >= 0 && hit.config < fc_wino_gemm_num_configs()) {
         printf("log entry exists.\n");
-        SetConfig(hit.config, hit.option);
-        printf("Best Config: (%zu %zu %zu) cfg=%d imgb=%d time=%.3f\n", input_channels, output_channels, input_width,
-               gemmConfig_best, imgBlock_best, hit.ms);
+        // option = 2 * images per block + offline flag
+        SetConfig(hit.config, hit.option / 2);
+        enableOffKernel_best = hit.option % 2;
+        printf("Best Config: (%zu %zu %zu) cfg=%d imgb=%d eoffK%d time=%.3f\n", input_channels, output_channels, input_width,
+               gemmConfig_best, imgBlock_best, enableOffKernel_best, hit.ms);
         return -1;
     }
     printf("log entry doesn't exist.\n");
@@ -152,6 +162,7 @@ int ConvWinoF63Layer::Tuning() {
             size_t cap, used, peak;
             fc_pool_stats(d.pool(), &cap, &used, &peak);
             if (probe.U_bytes + probe.V_bytes + 4096 > cap - used) continue;
+          for (enableOffKernel = 1; enableOffKernel >= 0; enableOffKernel--) {
             const size_t mark = d.Mark();
             AllocateFor(cfg, ib);
             RunOnce();
@@ -168,22 +179,24 @@ int ConvWinoF63Layer::Tuning() {
                 dev.Download(output_data, output_elements());
                 dis = diff(output_ref, output_data, (int)output_elements());
             }
-            printf("ocb=%d tb=%d icb=%d ocr%d tbr%d cfg=%d imgb=%d time=%.3f, diff=%.3f\n", ocBlock, tileBlock, icBlock,
-                   ocRegBlock, tileRegBlock, cfg, ib, elapsedTime, dis);
+            printf("ocb=%d tb=%d icb=%d ocr%d tbr%d cfg=%d imgb=%d eoffK%d time=%.3f, diff=%.3f\n", ocBlock, tileBlock,
+                   icBlock, ocRegBlock, tileRegBlock, cfg, ib, enableOffKernel, elapsedTime, dis);
             if (minTimeusage > elapsedTime) {
                 gemmConfig_best = cfg;
                 imgBlock_best = ib;
+                enableOffKernel_best = enableOffKernel;
                 minTimeusage = elapsedTime;
             }
             d.Release(mark);
             inputBuf = gemmBuf = kernelBuf = NULL;
+          }
         }
     }
     dev.Release();
-    TuningEntry e = {gemmConfig_best, imgBlock_best, minTimeusage};
+    TuningEntry e = {gemmConfig_best, 2 * imgBlock_best + enableOffKernel_best, minTimeusage};
     tuning_log_append(key, e);
-    printf("Best Config: (%zu %zu %zu) cfg=%d imgb=%d time=%.3f\n", input_channels, output_channels, input_width,
-           gemmConfig_best, imgBlock_best, minTimeusage);
+    printf("Best Config: (%zu %zu %zu) cfg=%d imgb=%d eoffK%d time=%.3f\n", input_channels, output_channels, input_width,
+           gemmConfig_best, imgBlock_best, enableOffKernel_best, minTimeusage);
     return -1;
 }
 
@@ -191,8 +204,10 @@ int ConvWinoF63Layer::Init() {
     const size_t in_elems = batch * input_channels * input_height * input_width;
     dev.Acquire(input_data, in_elems, kernel_data, output_channels * input_channels * 9, output_elements());
     if (channel_bias) dev.SetBias(channel_bias, output_channels);
+    enableOffKernel = enableOffKernel_best;
     AllocateFor(gemmConfig_best, imgBlock_best);
     printf("Algorithm: winograd F63 (blocked%s)\n", onePass ? ", single kernel" : "");
+    if (enableOffKernel) printf("offline kernel transform.\n");
     printf("enableoffkernel = %d\n", enableOffKernel);
     printf("Testing ic=%zu oc=%zu width=%zu batch=%zu tileBlock=%d (%d images) ocBlock=%d icBlock=%d\n", input_channels,
            output_channels, input_width, batch, tileBlock, imgBlock, ocBlock, icBlock);
@@ -218,7 +233,7 @@ int ConvWinoF63Layer::Forward() {
 
     d.Check(fc_timing_enable(d.ctx(), FC_TIMING_ALL), "fc_timing_enable");
     d.Check(fc_timing_reset(d.ctx()), "fc_timing_reset");
-    for (size_t i = 0; i < iterations; i++) RunOnce();
+    for (size_t i = 0; i < iterations; i++) RunOnce(true);
     // the GEMM and the output transform are one kernel here: its time is listed as TensorGEMM
     // (with the single-kernel engine that one kernel also holds the input transform)
     const int stages[4] = {FC_STAGE_INPUT_TRAN, FC_STAGE_KERNEL_TRAN, onePass ? FC_STAGE_ONEPASS : FC_STAGE_FUSED_GEMM_OUT,

@@ -2,8 +2,9 @@
 // (32 output channels x 32 tiles x 64 frequencies) is consumed by the output
 // transform straight out of registers and LDS -- there is no whole-layer M
 // buffer -- and the batch may be cut into blocks of `tileBlock` tiles (whole
-// images) so that only one block of V exists at a time.  The filter transform is
-// always done once in Init().  Interface of the reference's ConvWinoF63Layer
+// images) so that only one block of V exists at a time.  The filter transform runs
+// in every Forward() pass (online, the default) or once in Init() (offline:
+// SetConfig(..., 1), or chosen by Tuning()).  Interface of the reference's ConvWinoF63Layer
 // (convLayer/winoF63Conv.h:4-209), whose scratch is likewise sized for one
 // (ocBlock x tileBlock) block and whose GEMM output goes to the output
 // transform through a small buffer (winoF63/winoF63.cpp:1574-1737).
@@ -31,7 +32,9 @@ class ConvWinoF63Layer : public ConvLayer {
     // Not in the reference: fix tile shape and images per block by hand (0 images per block: the
     // single-kernel engine over the whole batch).
     void SetConfig(int gemm_config, int images_per_block);
+    void SetOfflineKernelTransform(bool offline) { enableOffKernel_best = offline ? 1 : 0; }
     int best_config() const { return gemmConfig_best; }
+    int best_offline() const { return enableOffKernel_best; }
     int best_images_per_block() const { return imgBlock_best; }
     double stage_ms[4] = {0, 0, 0, 0};
 
@@ -41,7 +44,7 @@ class ConvWinoF63Layer : public ConvLayer {
    private:
     fc_conv_shape Shape(int n) const;
     void AllocateFor(int config, int images_per_block);
-    void RunOnce();
+    void RunOnce(bool split_stages = false);
 
     int tileBlock;   // tiles per block = images per block x tiles per image
     int ocBlock;     // BM of the GEMM tile
@@ -57,6 +60,7 @@ class ConvWinoF63Layer : public ConvLayer {
 
     int gemmConfig_best;
     int imgBlock_best;
+    int enableOffKernel_best;
 
     fc_wino_plan plan, tailPlan;   // full blocks / the last partial block
     bool hasTail;

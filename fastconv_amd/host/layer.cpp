@@ -11,6 +11,15 @@ namespace feather {
 
 static size_t round256(size_t v) { return (v + 255) / 256 * 256; }
 
+// Init() and Forward() return int with 0 = success (the pools report failure as `false`).
+#define POOL_OK_OR_FAIL(call)                                                \
+    do {                                                                     \
+        if (!(call)) {                                                       \
+            fprintf(stderr, "Err in file %s line %d\n", __FILE__, __LINE__); \
+            return -1;                                                       \
+        }                                                                    \
+    } while (0)
+
 int ConvolutionLayer::GenerateTopBlobs() {
     const Blob<float> *in = _bottom_blobs[_bottom[0]];
     shape_.N = (int)in->num(); shape_.C = (int)in->channels(); shape_.H = (int)in->height(); shape_.W = (int)in->width();
@@ -24,10 +33,10 @@ int ConvolutionLayer::GenerateTopBlobs() {
 int ConvolutionLayer::Init() {
     Device &d = Device::Get();
     const size_t w_elems = oc_ * shape_.C * k_ * k_;
-    MEMPOOL_CHECK_RETURN(private_mempool->Alloc(&w_dev_, w_elems * sizeof(float)));
+    POOL_OK_OR_FAIL(private_mempool->Alloc(&w_dev_, w_elems * sizeof(float)));
     d.Check(fc_upload(d.ctx(), w_dev_, w_host_, w_elems * sizeof(float)), "upload weights");
     if (b_host_) {
-        MEMPOOL_CHECK_RETURN(private_mempool->Alloc(&b_dev_, oc_ * sizeof(float)));
+        POOL_OK_OR_FAIL(private_mempool->Alloc(&b_dev_, oc_ * sizeof(float)));
         d.Check(fc_upload(d.ctx(), b_dev_, b_host_, oc_ * sizeof(float)), "upload bias");
     }
     nnp_size ks = {k_, k_}, st = {s_, s_}, os = {_top_blobs[_name]->width(), _top_blobs[_name]->height()};
@@ -37,12 +46,12 @@ int ConvolutionLayer::Init() {
     if (onepass_) {
         // the whole layer in one kernel: no shared scratch at all
         d.Check(fc_wino_make_onepass_plan(&shape_, &wplan_), "fc_wino_make_onepass_plan");
-        MEMPOOL_CHECK_RETURN(private_mempool->Alloc(&U_, wplan_.U_bytes));
+        POOL_OK_OR_FAIL(private_mempool->Alloc(&U_, wplan_.U_bytes));
         d.Check(fc_wino_onepass_filter_transform(d.ctx(), &wplan_, w_dev_, U_), "fc_wino_onepass_filter_transform");
     } else if (winograd_) {
         d.Check(fc_wino_make_plan(&shape_, fc_wino_gemm_default_config(&shape_), &wplan_), "fc_wino_make_plan");
         fused_ = fc_wino_prefer_fused(&shape_) != 0;
-        MEMPOOL_CHECK_RETURN(private_mempool->Alloc(&U_, wplan_.U_bytes));
+        POOL_OK_OR_FAIL(private_mempool->Alloc(&U_, wplan_.U_bytes));
         // weights are constant: the filter transform is done once, here
         d.Check(fc_wino_filter_transform(d.ctx(), &wplan_, w_dev_, U_), "fc_wino_filter_transform");
         v_off_ = 0;
@@ -50,9 +59,9 @@ int ConvolutionLayer::Init() {
         common_mempool->Request(m_off_ + (fused_ ? 0 : wplan_.M_bytes));
     } else {
         d.Check(fc_igemm_make_plan(&shape_, fc_igemm_default_config(&shape_), &iplan_), "fc_igemm_make_plan");
-        MEMPOOL_CHECK_RETURN(private_mempool->Alloc(&Wp_, iplan_.Wp_bytes));
+        POOL_OK_OR_FAIL(private_mempool->Alloc(&Wp_, iplan_.Wp_bytes));
         float *tab = NULL;
-        MEMPOOL_CHECK_RETURN(private_mempool->Alloc(&tab, iplan_.table_bytes));
+        POOL_OK_OR_FAIL(private_mempool->Alloc(&tab, iplan_.table_bytes));
         table_ = (int32_t *)tab;
         d.Check(fc_igemm_pack_filter(d.ctx(), &iplan_, w_dev_, Wp_, table_), "fc_igemm_pack_filter");
         if (iplan_.ws_bytes) common_mempool->Request(iplan_.ws_bytes);
@@ -69,7 +78,7 @@ int ConvolutionLayer::Forward() {
         d.Check(fc_wino_conv_onepass(d.ctx(), &wplan_, x, U_, b_dev_, relu_, y), "fc_wino_conv_onepass");
         return 0;
     }
-    if (winograd_ || iplan_.ws_bytes) MEMPOOL_CHECK_RETURN(common_mempool->GetPtr(&scratch));
+    if (winograd_ || iplan_.ws_bytes) POOL_OK_OR_FAIL(common_mempool->GetPtr(&scratch));
     if (winograd_) {
         float *V = scratch, *M = (float *)((char *)scratch + m_off_);
         if (fused_)
@@ -99,6 +108,7 @@ int MaxPool2x2Layer::Forward() {
 
 Net::Net(size_t arena_bytes) : input_(NULL), graph_(NULL) {
     Device &d = Device::Get();
+    arena_mark_ = d.Mark();
     arena_block_ = d.Alloc(arena_bytes, "layer graph arena");
     alloc_ = new fastconv::RangeAllocator(arena_block_, arena_bytes, 256);
     common_ = new CommonMemPool<float>(alloc_);
@@ -110,6 +120,10 @@ Net::~Net() {
     delete input_;
     delete common_;
     delete alloc_;
+    // the device arena is a stack: the block goes back when nothing was allocated after it
+    Device &d = Device::Get();
+    size_t cap = 0, used = 0, peak = 0;
+    if (fc_pool_stats(d.pool(), &cap, &used, &peak) == FC_OK && used >= arena_mark_) d.Release(arena_mark_);
 }
 
 void Net::SetInput(size_t n, size_t c, size_t h, size_t w) {
@@ -154,9 +168,18 @@ int Net::RecordGraph() {
     if (Forward(NULL) != 0) return -1;      // every kernel has run once: LDS grants are in place
     d.Check(fc_sync(d.ctx()), "fc_sync");
     d.Check(fc_graph_begin(d.ctx()), "fc_graph_begin");
-    for (size_t i = 0; i < layers_.size(); i++)
-        if (layers_[i]->Forward() != 0) return -1;
-    d.Check(fc_graph_end(d.ctx(), &graph_), "fc_graph_end");
+    int failed = 0;
+    for (size_t i = 0; i < layers_.size() && !failed; i++) failed = layers_[i]->Forward() != 0;
+    // the recording is always closed, also when a layer refused: the stream must not stay in capture mode
+    fc_graph *g = NULL;
+    const int rc = fc_graph_end(d.ctx(), &g);
+    if (failed || rc != FC_OK) {
+        if (g) fc_graph_destroy(g);
+        fprintf(stderr, "Error: recording the layer graph failed%s%s\n", rc != FC_OK ? ": " : "",
+                rc != FC_OK ? fc_last_error(d.ctx()) : "");
+        return -1;
+    }
+    graph_ = g;
     return 0;
 }
 

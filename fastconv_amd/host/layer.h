@@ -74,7 +74,8 @@ class ConvolutionLayer : public Layer {
     ConvolutionLayer(const std::string &name, size_t oc, size_t kernel, size_t stride, size_t pad, const float *weights,
                      const float *bias, bool relu)
         : Layer(name, "Convolution"), oc_(oc), k_(kernel), s_(stride), p_(pad), w_host_(weights), b_host_(bias),
-          relu_(relu), winograd_(false), fused_(false), onepass_(false), w_dev_(NULL), b_dev_(NULL), U_(NULL), Wp_(NULL), table_(NULL) {}
+          relu_(relu), winograd_(false), fused_(false), onepass_(false), w_dev_(NULL), b_dev_(NULL), U_(NULL), Wp_(NULL), table_(NULL),
+          shape_(), wplan_(), iplan_(), v_off_(0), m_off_(0) {}
 
     int GenerateTopBlobs();
     int Init();
@@ -124,6 +125,7 @@ class Net {
     Blob<float> *input_;
     std::vector<Layer *> layers_;
     void *arena_block_;
+    size_t arena_mark_;
     fc_graph *graph_;
 };
 

@@ -1,13 +1,13 @@
 // Algorithm choice for `-a auto`.  The reference picks by kernel size and
 // stride alone (ConvTest.cpp:318-331: 1x1 stride 1 -> direct, 3x3 stride 1 ->
-// winograd, otherwise im2col).  The same skeleton is kept, with the 3x3
-// stride-1 case refined by what was measured on MI355X: the staged Winograd
-// pipeline moves 64 planes of V and M per layer, which only pays when there is
-// enough arithmetic per plane element.
+// winograd, otherwise im2col).  The same skeleton is kept; the 3x3 stride-1 case
+// asks the kernel library, whose rule (fc_prefer_winograd) is derived from
+// measured per-layer times of both paths on MI355X.
 #pragma once
 
 #include <algorithm>
 
+#include "fastconv_hip.h"
 #include "utility/helper.h"
 
 inline enum nnp_convolution_algorithm select_algorithm(struct nnp_size kernel_size, struct nnp_size output_subsampling,
@@ -17,12 +17,10 @@ inline enum nnp_convolution_algorithm select_algorithm(struct nnp_size kernel_si
         if (std::max(kernel_size.height, kernel_size.width) == 1) {
             return nnp_convolution_algorithm_direct;
         } else if (kernel_size.height == 3 && kernel_size.width == 3) {
-            const size_t tiles = batch * ((output_size.height + 5) / 6) * ((output_size.width + 5) / 6);
-            // few input channels: the M planes (64 floats per 36 outputs) dominate and carry no reuse
-            if (input_channels < 16) return nnp_convolution_algorithm_im2col;
-            // few tiles: the 64x larger transformed filter dominates
-            if (tiles < 64 && input_channels * output_channels >= 128 * 128) return nnp_convolution_algorithm_im2col;
-            return nnp_convolution_algorithm_winograd;
+            // the rule sees the layer through its output size: an input of the same size with padding 1
+            fc_conv_shape s = {(int)batch, (int)input_channels, (int)output_size.height, (int)output_size.width,
+                               (int)output_channels, 3, 3, 1, 1, 1, 1, 1, 1};
+            return fc_prefer_winograd(&s) ? nnp_convolution_algorithm_winograd : nnp_convolution_algorithm_im2col;
         }
     }
     return nnp_convolution_algorithm_im2col;

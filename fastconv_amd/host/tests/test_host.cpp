@@ -156,7 +156,39 @@ static void test_rng() {
     }
 }
 
-int main() {
+// `test_host --naive in.bin out.bin`: runs the host ConvNaiveLayer on a case read from in.bin
+// (13 int32 of geometry N,C,H,W,K,kh,kw,sh,sw,pt,pb,pl,pr, one int32 "has per-element bias",
+// then x, w and the optional bias as float32) and writes the output as float32, so that a
+// test can compare its bits with stored results of the reference's own naive layers.
+static int run_naive_case(const char *in_path, const char *out_path) {
+    FILE *f = fopen(in_path, "rb");
+    if (!f) return 2;
+    int g[14];
+    if (fread(g, sizeof(int), 14, f) != 14) return 2;
+    const size_t N = g[0], C = g[1], H = g[2], W = g[3], K = g[4], kh = g[5], kw = g[6];
+    const size_t nx = N * C * H * W, nw = K * C * kh * kw;
+    const size_t OH = (H + g[9] + g[10] - kh) / g[7] + 1, OW = (W + g[11] + g[12] - kw) / g[8] + 1;
+    float *x = (float *)malloc(sizeof(float) * nx), *w = (float *)malloc(sizeof(float) * nw), *b = NULL;
+    if (fread(x, sizeof(float), nx, f) != nx || fread(w, sizeof(float), nw, f) != nw) return 2;
+    if (g[13]) {
+        b = (float *)malloc(sizeof(float) * K * OH * OW);
+        if (fread(b, sizeof(float), K * OH * OW, f) != K * OH * OW) return 2;
+    }
+    fclose(f);
+    ConvNaiveLayer layer(x, w, b, NULL, C, H, W, K, kh, kw, g[7], g[8], g[11], g[12], g[9], g[10], 1, b != NULL, 2, 1, N);
+    layer.Forward();
+    FILE *o = fopen(out_path, "wb");
+    if (!o) return 2;
+    fwrite(layer.output_data, sizeof(float), layer.output_elements(), o);
+    fclose(o);
+    free(x);
+    free(w);
+    free(b);
+    return 0;
+}
+
+int main(int argc, char **argv) {
+    if (argc == 4 && strcmp(argv[1], "--naive") == 0) return run_naive_case(argv[2], argv[3]);
     test_range_allocator();
     test_pools();
     test_tuning_log();

@@ -7,13 +7,14 @@
 #include <string>
 
 struct TuningKey {
-    const char *algo;   // "winograd_zc", "winograd", "im2col"
+    const char *algo;   // "winograd_zc", "winograd_blocked", "im2col"
     int n, c, h, w, k, kh, kw, sh, sw, pt, pb, pl, pr;
 };
 
 struct TuningEntry {
     int config;      // tile-shape id of the GEMM stage / implicit GEMM
-    int option;      // algorithm specific: filter transform offline (1) / online (0); images per block
+    int option;      // winograd_zc: filter transform offline (1) / online (0);
+                     // winograd_blocked: 2 * images per block + the same flag; im2col: unused
     double ms;       // best time per Forward
 };
 

@@ -170,7 +170,18 @@ typedef struct {
     size_t U_bytes, V_bytes, M_bytes;
 } fc_wino_plan;
 
+/* FC_ERR_INVALID unless the layer is 3x3 with stride 1; FC_ERR_UNSUPPORTED when the output is
+ * wider than 1020 columns (170 tiles: two bands of the input transform must fit 64 KiB of LDS)
+ * or a buffer would pass 2^31 elements per frequency plane.  Every later call checks the plan it
+ * is given against the one this function makes for plan->shape and plan->gemm_config. */
 int fc_wino_make_plan(const fc_conv_shape *shape, int gemm_config, fc_wino_plan *plan);
+
+/* The rule behind `-a auto` for one layer (select_algorithm, ConvTest.cpp:318-331, which looks at
+ * filter size and stride only): 1 when the Winograd path is expected to be faster than the
+ * implicit GEMM on MI355X, 0 when not or when Winograd cannot run the layer at all (not 3x3
+ * stride 1, or wider than fc_wino_make_plan admits).  The thresholds come from measured
+ * per-layer times of both paths on the VGG-16 and ResNet-50 layers at batch 1 and 32. */
+int fc_prefer_winograd(const fc_conv_shape *shape);
 
 /* U = G g G^T.  Replaces the kernel transform inside winoF63_v1_single
  * (winoF63ZC/winoF63ZC.cpp:433-500) and offline_kernel_transform_v1 (:242-322).

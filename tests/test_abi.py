@@ -73,6 +73,18 @@ def test_plans_are_pure_host_arithmetic():
     assert (q.Kred_pad // 16) >= 4 * q.split_k
 
 
+def test_winograd_width_limit_is_part_of_the_plan_and_of_the_auto_rule():
+    lib = capi.load_cdll()
+    p = capi.WinoPlan()
+    ok = capi.ConvShape(1, 64, 9, 1020, 64, 3, 3, 1, 1, 1, 1, 1, 1)
+    wide = capi.ConvShape(1, 64, 9, 1021, 64, 3, 3, 1, 1, 1, 1, 1, 1)
+    assert lib.fc_wino_make_plan(C.byref(ok), 0, C.byref(p)) == 0 and p.tiles_w == 170
+    assert lib.fc_wino_make_plan(C.byref(wide), 0, C.byref(p)) == -6
+    assert lib.fc_prefer_winograd(C.byref(ok)) == 1 and lib.fc_prefer_winograd(C.byref(wide)) == 0
+    strided = capi.ConvShape(1, 64, 56, 56, 64, 3, 3, 2, 2, 1, 1, 1, 1)
+    assert lib.fc_prefer_winograd(C.byref(strided)) == 0
+
+
 def test_no_gpu_means_a_loud_error_not_a_fallback():
     import pytest
     lib = capi.load_cdll()
@@ -84,3 +96,31 @@ def test_no_gpu_means_a_loud_error_not_a_fallback():
     assert rc == -2 and not ctx.value
     with pytest.raises(capi.FastConvError):
         capi.Library(0)
+
+
+def test_struct_layouts_match_the_header(tmp_path):
+    """sizeof and every field offset of the ctypes structures against what a C compiler makes of
+    include/fastconv_hip.h."""
+    import subprocess
+    structs = {"fc_conv_shape": capi.ConvShape, "fc_gemm_config": capi.GemmConfig, "fc_wino_plan": capi.WinoPlan,
+               "fc_igemm_plan": capi.IgemmPlan, "fc_device_info": capi.DeviceInfo}
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "fastconv_hip.h"', 'int main(void) {']
+    for cname, ct in structs.items():
+        lines.append('printf("%s sizeof %%zu\\n", sizeof(%s));' % (cname, cname))
+        for fname, _ in ct._fields_:
+            lines.append('printf("%s %s %%zu\\n", offsetof(%s, %s));' % (cname, fname, cname, fname))
+    lines += ['return 0;', '}']
+    src, exe = tmp_path / "layout.c", tmp_path / "layout"
+    src.write_text("\n".join(lines))
+    subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)])
+    seen = 0
+    for line in subprocess.check_output([str(exe)], text=True).splitlines():
+        cname, field, value = line.split()
+        ct = structs[cname]
+        if field == "sizeof":
+            assert C.sizeof(ct) == int(value), cname
+        else:
+            assert getattr(ct, field).offset == int(value), (cname, field)
+        seen += 1
+    assert seen == sum(len(ct._fields_) + 1 for ct in structs.values())
+    assert len(capi.STAGE_NAMES) == 8       # FC_STAGE_COUNT

@@ -38,6 +38,63 @@ def test_conv_test_driver_passes_its_own_check(algo):
     assert "PASS" in out and "FAIL" not in out
 
 
+def _json_line(out):
+    import json
+    return json.loads([l for l in out.splitlines() if l.startswith("{")][-1])
+
+
+@pytest.mark.parametrize("variant", ["zc", "blocked"])
+@pytest.mark.parametrize("batch,C,H", [(64, 256, 56), (128, 256, 56), (64, 512, 28), (128, 512, 28), (64, 512, 14),
+                                       (128, 512, 14)])
+def test_stress_layers_through_both_winograd_layer_classes_with_tuning(tmp_path, variant, batch, C, H):
+    """Batch 64 / 128 on the throughput-stress layers through ConvWinoF63ZCLayer (staged, whole-layer
+    buffers) and ConvWinoF63Layer (blocked) with -tn tuning; the driver's own check covers the last
+    image of the batch (the host convolution of 128 images would take minutes)."""
+    out = _run([_exe("conv_test"), "-ic", str(C), "-oc", str(C), "-is", str(H), str(H), "-ks", "3", "3", "-ip", "1",
+                "-n", str(batch), "-i", "2", "-t", "16", "-a", "winograd", "--variant", variant, "-tn", "tuning",
+                "--check-images", "1", "--strict", "--json"], cwd=str(tmp_path))
+    assert "PASS" in out and "FAIL" not in out and "Best Config" in out
+    j = _json_line(out)
+    assert j["batch"] == batch and j["checked_images"] == 1 and j["max_rel_err"] <= 1e-3
+    assert j["algorithm"] == ("winograd_blocked" if variant == "blocked" else "winograd")
+    assert j["kernel_transform"] in ("online", "offline")
+
+
+@pytest.mark.parametrize("geo", [
+    # ResNet-50 (run_resnet50.sh:10-30 and the 3x3 stride-2 variant): ic, oc, size, kernel, stride, pad
+    (64, 64, 56, 3, 1, 1), (128, 128, 28, 3, 1, 1), (256, 256, 14, 3, 1, 1), (512, 512, 7, 3, 1, 1),
+    (256, 64, 56, 1, 1, 0), (64, 256, 56, 1, 1, 0), (512, 128, 28, 1, 1, 0), (1024, 256, 14, 1, 1, 0),
+    (2048, 512, 7, 1, 1, 0), (128, 128, 56, 3, 2, 1), (3, 64, 224, 7, 2, 3)])
+@pytest.mark.parametrize("batch", [1, 32])
+def test_auto_algorithm_on_resnet50_layers(geo, batch):
+    ic, oc, size, ks, st, pad = geo
+    out = _run([_exe("conv_test"), "-ic", str(ic), "-oc", str(oc), "-is", str(size), str(size), "-ks", str(ks), str(ks),
+                "-s", str(st), str(st), "-ip", str(pad), "-n", str(batch), "-i", "2", "-t", "16", "-a", "auto",
+                "--check-images", "1", "--strict", "--json"])
+    assert "PASS" in out and "FAIL" not in out
+    j = _json_line(out)
+    # the driver's choice is the library's rule (3x3 stride 1) inside the reference's skeleton
+    from fastconv_amd import capi
+    import ctypes
+    shape = capi.ConvShape(batch, ic, size, size, oc, ks, ks, st, st, pad, pad, pad, pad)
+    want = "winograd" if capi.load_cdll().fc_prefer_winograd(ctypes.byref(shape)) else "im2col"
+    if ks == 1 and st == 1:
+        want = "direct"
+    if batch == 32 and ks == 3 and st == 1:
+        assert want == "winograd"
+    assert j["algorithm"].split("_")[0] == want, j
+    assert j["max_rel_err"] <= (1e-3 if want == "winograd" else 1e-5)
+
+
+def test_blocked_variant_honours_the_transform_strategy():
+    base = [_exe("conv_test"), "-ic", "16", "-oc", "24", "-is", "28", "28", "-ks", "3", "3", "-n", "2", "-i", "2",
+            "--strict", "--json", "-a", "winograd", "--variant", "blocked"]
+    on = _json_line(_run(base))
+    off = _json_line(_run(base + ["-ts", "offline"]))
+    assert on["kernel_transform"] == "online" and off["kernel_transform"] == "offline"
+    assert on["kernel_tran_ms"] > 0.0 and off["kernel_tran_ms"] == 0.0
+
+
 def test_conv_test_pointwise_and_strided_go_to_implicit_gemm():
     out = _run([_exe("conv_test"), "-ic", "32", "-oc", "16", "-is", "14", "14", "-ks", "1", "1", "-a", "auto",
                 "-i", "2", "--strict"])

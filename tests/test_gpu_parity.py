@@ -85,6 +85,48 @@ def test_winograd_against_oracle(lib, shp):
     assert O.max_rel_err(y, O.wino_conv_f32(s, x, w)) <= 1e-4
 
 
+# every 3x3 stride-1 layer of VGG-16 (run_vgg16.sh:5-13) and ResNet-50 (run_resnet50.sh:10-30): (C, K, H)
+VGG16_3X3 = [(3, 64, 224), (64, 64, 224), (64, 128, 112), (128, 128, 112), (128, 256, 56), (256, 256, 56),
+             (256, 512, 28), (512, 512, 28), (512, 512, 14)]
+RESNET50_3X3 = [(64, 64, 56), (128, 128, 28), (256, 256, 14), (512, 512, 7)]
+
+
+@pytest.mark.parametrize("C,K,H", VGG16_3X3 + RESNET50_3X3)
+def test_batch1_real_layers_every_path_against_oracle(lib, C, K, H):
+    """Batch 1 at the real channel counts: the staged, fused and single-kernel Winograd
+    pipelines (<= 1e-3) and the implicit GEMM (<= 1e-5) against the fp64 direct convolution."""
+    s = O.shape(1, C, H, H, K)
+    cs = cshape(s)
+    x, w = O.make_inputs(s, seed=0)
+    announce("batch-1 real layer", (C, K, H))
+    truth = O.naive_conv_f64(s, x, w)
+    assert O.max_rel_err(lib.implicit_gemm_conv(cs, x, w), truth) <= TOL_IM2COL
+    assert O.max_rel_err(lib.winograd_conv(cs, x, w), truth) <= TOL_WINO
+    assert O.max_rel_err(lib.winograd_conv_fused(cs, x, w), truth) <= TOL_WINO
+    if H >= 8:          # a patch row of the single-kernel path is 8 floats of one image row
+        assert O.max_rel_err(lib.winograd_conv_onepass(cs, x, w), truth) <= TOL_WINO
+
+
+def test_winograd_wide_images(lib):
+    """Outputs up to 1020 columns (170 tiles per band) are inside the stated limit of the staged
+    pipeline; 512 and 1020 columns take the narrower blocks of the input transform."""
+    import fastconv_amd as F
+    for (N, C, H, W, K) in [(1, 3, 20, 512, 4), (1, 2, 9, 1020, 3), (2, 5, 14, 640, 6), (1, 4, 7, 760, 2)]:
+        s = O.shape(N, C, H, W, K)
+        x, w = O.make_inputs(s, seed=W)
+        truth = O.naive_conv_f64(s, x, w)
+        for cfg in (0, 3, 4):
+            announce("wide image", (N, C, H, W, K), "cfg", cfg)
+            assert O.max_rel_err(lib.winograd_conv(cshape(s), x, w, config=cfg), truth) <= TOL_WINO
+        assert O.max_rel_err(lib.winograd_conv_fused(cshape(s), x, w), truth) <= TOL_WINO
+        assert O.max_rel_err(lib.winograd_conv_onepass(cshape(s), x, w), truth) <= TOL_WINO
+        assert lib.prefer_winograd(cshape(O.shape(N, 64, H, W, 64)))
+    with pytest.raises(F.FastConvError) as e:
+        lib.wino_plan(cshape(O.shape(1, 2, 9, 1021, 3)), 0)
+    assert e.value.status == -6
+    assert not lib.prefer_winograd(cshape(O.shape(1, 64, 9, 1021, 64)))     # auto falls back to implicit GEMM
+
+
 def test_winograd_every_tile_config(lib):
     s = O.shape(2, 40, 28, 28, 72)
     x, w = O.make_inputs(s, seed=5)
@@ -277,6 +319,10 @@ IGEMM_SHAPES = [
     # windows that never leave the image (no padding, whole-stage reduction): the gather without bounds masks
     (3, 32, 15, 15, 64, 1, 1, 2, 2, 0), (2, 16, 12, 13, 40, 3, 3, 1, 1, 0), (2, 48, 9, 9, 70, 1, 1, 1, 1, 0),
     (3, 4, 17, 16, 33, 2, 2, 2, 2, 0), (32, 256, 56, 56, 512, 1, 1, 2, 2, 0),
+    # ResNet-50 bottleneck layers at batch 32: 1x1 reduce / expand, 3x3 stride 2 (first layer of a stage), the stem
+    (32, 256, 56, 56, 64, 1, 1, 1, 1, 0), (32, 512, 28, 28, 128, 1, 1, 1, 1, 0), (32, 2048, 7, 7, 512, 1, 1, 1, 1, 0),
+    (32, 1024, 14, 14, 256, 1, 1, 1, 1, 0), (32, 128, 56, 56, 128, 3, 3, 2, 2, 1), (32, 256, 28, 28, 256, 3, 3, 2, 2, 1),
+    (32, 512, 14, 14, 512, 3, 3, 2, 2, 1), (8, 3, 224, 224, 64, 7, 7, 2, 2, 3),
 ]
 
 
@@ -368,8 +414,9 @@ def test_golden_vectors_of_reference_naive_layers(lib):
 
 def _full_layers():
     # (N, C, H, K): VGG-16 and ResNet-50 3x3 stride-1 layers at batch 32
-    return [(32, 3, 224, 64), (32, 64, 224, 64), (32, 128, 112, 128), (32, 256, 56, 256),
-            (32, 512, 28, 512), (32, 512, 14, 512), (32, 64, 56, 64), (32, 512, 7, 512)]
+    return [(32, 3, 224, 64), (32, 64, 224, 64), (32, 64, 112, 128), (32, 128, 112, 128), (32, 128, 56, 256),
+            (32, 256, 56, 256), (32, 256, 28, 512), (32, 512, 28, 512), (32, 512, 14, 512),
+            (32, 64, 56, 64), (32, 128, 28, 128), (32, 256, 14, 256), (32, 512, 7, 512)]
 
 
 @pytest.mark.parametrize("N,C,H,K", _full_layers())
@@ -390,7 +437,8 @@ def test_full_size_shift_kernel_property(lib, N, C, H, K):
     assert np.array_equal(yi, expect)            # one non-zero product per output: exact
 
 
-@pytest.mark.parametrize("N,C,H,K", [(32, 256, 56, 256), (32, 64, 224, 64), (32, 512, 14, 512)])
+@pytest.mark.parametrize("N,C,H,K", [(32, 256, 56, 256), (32, 64, 224, 64), (32, 512, 14, 512), (32, 128, 56, 256),
+                                     (32, 256, 28, 512), (32, 128, 28, 128), (32, 256, 14, 256)])
 def test_full_size_two_algorithms_agree_and_are_linear(lib, N, C, H, K):
     s = O.shape(N, C, H, H, K)
     x, w = O.make_inputs(s, seed=1)
@@ -420,6 +468,41 @@ def test_all_ones_closed_form_full_size(lib):
     assert np.array_equal(yi, expect)
     yw = lib.winograd_conv(cshape(s), x, w)
     assert O.max_rel_err(yw, expect) <= TOL_WINO
+
+
+# ------------------------------------------- large batches (64 and 128 images)
+
+@pytest.mark.parametrize("N", [64, 128])
+@pytest.mark.parametrize("C,H", [(256, 56), (512, 28), (512, 14)])
+def test_large_batch_stress_layers(lib, N, C, H):
+    """The throughput-stress layers at batch 64 and 128, through the staged pipeline (whole-layer
+    U, V, M), the blocked one (no M) and the implicit GEMM: an exact shift-kernel answer, agreement
+    of the three paths on seeded data, and the first and last image against the fp64 oracle."""
+    K = C
+    s = O.shape(N, C, H, H, K)
+    cs = cshape(s)
+    announce("stress layer", (N, C, H, K))
+    x = O.rng_uniform(21, (N, C, H, H))
+    u, v = 0, 2
+    wd = np.zeros((K, C, 3, 3), np.float32)
+    wd[np.arange(K), (np.arange(K) * 7 + 3) % C, u, v] = 1.0
+    xp = np.pad(x, ((0, 0), (0, 0), (1, 1), (1, 1)))
+    expect = xp[:, (np.arange(K) * 7 + 3) % C, u:u + H, v:v + H]
+    assert np.array_equal(lib.implicit_gemm_conv(cs, x, wd), expect)
+    assert O.max_rel_err(lib.winograd_conv(cs, x, wd), expect) <= TOL_WINO
+    assert O.max_rel_err(lib.winograd_conv_fused(cs, x, wd), expect) <= TOL_WINO
+    del xp, expect
+    _, w = O.make_inputs(O.shape(1, C, H, H, K), seed=4)
+    yi = lib.implicit_gemm_conv(cs, x, w)
+    ys = lib.winograd_conv(cs, x, w)
+    assert O.max_rel_err(ys, yi) <= TOL_WINO
+    yb = lib.winograd_conv_fused(cs, x, w)
+    assert np.array_equal(yb, ys)          # same products in the same order, M kept in registers instead of HBM
+    sub = O.shape(1, C, H, H, K)
+    for n in (0, N - 1):
+        truth = O.naive_conv_f64(sub, np.ascontiguousarray(x[n:n + 1]), w)
+        assert O.max_rel_err(yi[n:n + 1], truth) <= TOL_IM2COL
+        assert O.max_rel_err(ys[n:n + 1], truth) <= TOL_WINO
 
 
 # ------------------------------------------------------- recorded sequences

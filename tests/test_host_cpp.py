@@ -34,6 +34,30 @@ def test_driver_generator_matches_oracle_generator_bit_for_bit():
     assert np.array_equal(np.array(g, np.float32), O.rng_normal(7, (1001,), 0.5)[:8])
 
 
+def test_host_naive_layer_reproduces_the_reference_naive_layers_bit_for_bit(tmp_path):
+    """host/convLayer/naiveConv.h is the checker of conv_test and net_test: on every stored
+    case of the reference's own ConvNaiveLayers (tests/golden/naive_ref_vectors.npz) it
+    must give the same bits."""
+    exe = _build()
+    z = np.load(os.path.join(ROOT, "tests", "golden", "naive_ref_vectors.npz"))
+    names = sorted({k.split("/")[0] for k in z.files})
+    assert len(names) >= 10
+    for name in names:
+        has_bias = name + "/bias_elems" in z.files
+        src, dst = tmp_path / (name + ".in"), tmp_path / (name + ".out")
+        with open(src, "wb") as f:
+            f.write(z[name + "/shape"].astype(np.int32).tobytes())
+            f.write(np.int32(1 if has_bias else 0).tobytes())
+            f.write(np.ascontiguousarray(z[name + "/x"], np.float32).tobytes())
+            f.write(np.ascontiguousarray(z[name + "/w"], np.float32).tobytes())
+            if has_bias:
+                f.write(np.ascontiguousarray(z[name + "/bias_elems"], np.float32).tobytes())
+        r = subprocess.run([exe, "--naive", str(src), str(dst)], capture_output=True, text=True, timeout=60)
+        assert r.returncode == 0, (name, r.stderr)
+        y = np.fromfile(dst, np.float32).reshape(z[name + "/y"].shape)
+        assert np.array_equal(y, z[name + "/y"]), name
+
+
 def test_driver_refuses_to_run_without_a_gpu_or_reports_results():
     """conv_test has no CPU compute path: without a GPU it must stop with an error."""
     exe = os.path.join(PKG, "bin", "conv_test")
