@@ -112,7 +112,10 @@ _ABI = {
     "fc_igemm_make_plan": (C.c_int, [C.POINTER(ConvShape), C.c_int, C.POINTER(IgemmPlan)]),
     "fc_igemm_pack_filter": (C.c_int, [_vp, C.POINTER(IgemmPlan), _vp, _vp, _vp]),
     "fc_conv_implicit_gemm": (C.c_int, [_vp, C.POINTER(IgemmPlan), _vp, _vp, _vp, _vp, C.c_int, _vp, _vp]),
+    "fc_conv_implicit_gemm_static": (C.c_int, [_vp, C.POINTER(IgemmPlan), _vp, _vp, _vp, _vp, C.c_int, _vp]),
 }
+
+IGEMM_STATIC_WS_BYTES = 32 << 20
 
 
 def abi_symbols():
@@ -375,6 +378,10 @@ class Library:
 
     def conv_implicit_gemm(self, plan, x, Wp, table, y, bias=None, relu=False, ws=None):
         self._check(self.c.fc_conv_implicit_gemm(self.ctx, C.byref(plan), x, Wp, table, bias, int(relu), ws, y))
+
+    def conv_implicit_gemm_static(self, plan, x, Wp, table, y, bias=None, relu=False):
+        """As conv_implicit_gemm, with the split-reduction workspace inside the library (no allocation)."""
+        self._check(self.c.fc_conv_implicit_gemm_static(self.ctx, C.byref(plan), x, Wp, table, bias, int(relu), y))
 
     # ---- whole-layer helpers over host arrays (tests, smoke)
     def winograd_conv_fused(self, shape, x, w, bias=None, relu=False, config=None):

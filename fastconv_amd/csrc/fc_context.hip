@@ -65,6 +65,13 @@ extern "C" int fc_init(int device, fc_context **out) {
         return FC_ERR_NO_DEVICE;
     }
     if (hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking) != hipSuccess) { delete ctx; return FC_ERR_HIP; }
+    ctx->igemm_static_ws = nullptr;
+    if (fc_igemm_static_init(ctx) != FC_OK) {
+        fprintf(stderr, "fastconv: %s\n", ctx->last_error.c_str());
+        (void)hipStreamDestroy(ctx->stream);
+        delete ctx;
+        return FC_ERR_HIP;
+    }
     *out = ctx;
     return FC_OK;
 }
@@ -418,7 +425,7 @@ static hipEvent_t fc_take_event(fc_context *ctx) {
 }
 
 fc_stage_scope::fc_stage_scope(fc_context *c, int stage) : ctx(c), stop(nullptr), active(false) {
-    if (!(c->timing_mask & (1u << stage))) return;
+    if (stage < 0 || !(c->timing_mask & (1u << stage))) return;      // stage -1: never bracketed
     if (c->pending.size() >= 8192) (void)fc_timing_fold(c);
     hipEvent_t start = fc_take_event(c);
     stop = fc_take_event(c);

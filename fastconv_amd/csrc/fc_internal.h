@@ -31,6 +31,8 @@ struct fc_context {
     hipStream_t probe_stream;
     unsigned long long *probe_buf;
     int probe_samples;      // > 0 while a probe is running
+    // device address of the static split-reduction workspace of fc_conv_implicit_gemm_static
+    float *igemm_static_ws;
 };
 
 struct fc_graph {
@@ -52,6 +54,8 @@ static const uint32_t FC_POOL_MAGIC = 0x4643504cu;  // "FCPL"
 static const uint32_t FC_GRAPH_MAGIC = 0x46434752u; // "FCGR"
 
 int fc_set_error(fc_context *ctx, int status, const char *what, hipError_t err);
+// implicit_gemm.hip: looks up the static workspace of this context's device (once per device)
+int fc_igemm_static_init(fc_context *ctx);
 bool fc_ctx_ok(const fc_context *ctx);
 
 // Brackets one kernel launch with events when timing is on.

@@ -6,6 +6,8 @@
 // (output channel fastest) so that its tiles are straight 16-byte copies, as in
 // the Winograd GEMM.
 #include <cmath>
+#include <cstdio>
+#include <mutex>
 #include <utility>
 
 #include "fc_internal.h"
@@ -506,11 +508,66 @@ extern "C" int fc_igemm_pack_filter(fc_context *ctx, const fc_igemm_plan *plan, 
     return FC_OK;
 }
 
+// Launches of one layer; `timed` brackets the GEMM kernel with events when stage timing is on.
+static int igemm_run(fc_context *ctx, const fc_igemm_plan *plan, const float *x_dev, const float *Wp_dev,
+                     const int32_t *table_dev, const float *bias_dev, int relu, float *ws_dev, float *y_dev, bool timed);
+
 extern "C" int fc_conv_implicit_gemm(fc_context *ctx, const fc_igemm_plan *plan, const float *x_dev,
                                      const float *Wp_dev, const int32_t *table_dev, const float *bias_dev, int relu,
                                      float *ws_dev, float *y_dev) {
     const int rc = ig_plan_check(ctx, plan);
     if (rc) return rc;
+    return igemm_run(ctx, plan, x_dev, Wp_dev, table_dev, bias_dev, relu, ws_dev, y_dev, true);
+}
+
+// ---- the same layer with the split-reduction workspace in a static device array ----
+
+// Partial sums of a split reduction, [split][K][N*OH*OW] floats, for callers that cannot allocate.
+// Every GPU the library runs on holds its own copy of this array until the process ends.
+static __device__ __align__(256) float scratch[FC_IGEMM_STATIC_WS_BYTES / sizeof(float)];
+
+// Device address of `scratch` per device, looked up once per device with that device current.
+static const int kMaxDevices = 64;
+static float *g_scratch_ptr[kMaxDevices];
+static bool g_scratch_known[kMaxDevices];
+static std::mutex g_scratch_mutex;
+
+// Called by fc_init with ctx->device current.
+int fc_igemm_static_init(fc_context *ctx) {
+    if (ctx->device < 0 || ctx->device >= kMaxDevices)
+        return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_igemm_static_init: device index above 63", hipSuccess);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_known[ctx->device]) {
+        float *ptr = nullptr;
+        FC_HIP_CHECK(ctx, hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return fc_set_error(ctx, FC_ERR_HIP, "fc_igemm_static_init: null address of the static workspace", hipSuccess);
+        g_scratch_ptr[ctx->device] = ptr;
+        g_scratch_known[ctx->device] = true;
+    }
+    ctx->igemm_static_ws = g_scratch_ptr[ctx->device];
+    return FC_OK;
+}
+
+extern "C" int fc_conv_implicit_gemm_static(fc_context *ctx, const fc_igemm_plan *plan, const float *x_dev,
+                                            const float *Wp_dev, const int32_t *table_dev, const float *bias_dev,
+                                            int relu, float *y_dev) {
+    const int rc = ig_plan_check(ctx, plan);
+    if (rc) return rc;
+    if (plan->ws_bytes > (size_t)FC_IGEMM_STATIC_WS_BYTES) {
+        char msg[200];
+        snprintf(msg, sizeof msg, "fc_conv_implicit_gemm_static: this layer needs %zu bytes of split-reduction workspace, "
+                 "the static one holds %d: use fc_conv_implicit_gemm with a workspace of the caller's", plan->ws_bytes,
+                 FC_IGEMM_STATIC_WS_BYTES);
+        return fc_set_error(ctx, FC_ERR_UNSUPPORTED, msg, hipSuccess);
+    }
+    if (!ctx->igemm_static_ws) return fc_set_error(ctx, FC_ERR_STATE, "fc_conv_implicit_gemm_static: static workspace not set up", hipSuccess);
+    // Nothing has to start at zero: every partial sum the reduction reads ([split][k < K][pixel < Npix]) is
+    // written by this call's GEMM kernel first.  No event brackets (creating an event may allocate).
+    return igemm_run(ctx, plan, x_dev, Wp_dev, table_dev, bias_dev, relu, ctx->igemm_static_ws, y_dev, false);
+}
+
+static int igemm_run(fc_context *ctx, const fc_igemm_plan *plan, const float *x_dev, const float *Wp_dev,
+                     const int32_t *table_dev, const float *bias_dev, int relu, float *ws_dev, float *y_dev, bool timed) {
     if (!x_dev || !Wp_dev || !table_dev || !y_dev)
         return fc_set_error(ctx, FC_ERR_INVALID, "fc_conv_implicit_gemm: null buffer", hipSuccess);
     if ((uintptr_t)Wp_dev & 15) return fc_set_error(ctx, FC_ERR_INVALID, "fc_conv_implicit_gemm: Wp must be 16-byte aligned", hipSuccess);
@@ -534,7 +591,7 @@ extern "C" int fc_conv_implicit_gemm(fc_context *ctx, const fc_igemm_plan *plan,
     p.fastStore = s.K % cfg.bm == 0 && 4.0 * s.N * s.K * plan->OH * plan->OW < 4294967296.0 &&
                   4.0 * plan->split_k * s.K * (double)plan->Npix < 4294967296.0 && ((uintptr_t)bias_dev & 15) == 0;
     if ((long)p.nKB * p.nPB >= (1l << 31)) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_conv_implicit_gemm: grid too large", hipSuccess);
-    fc_stage_scope scope(ctx, FC_STAGE_IMPLICIT_GEMM);
+    fc_stage_scope scope(ctx, timed ? FC_STAGE_IMPLICIT_GEMM : -1);
     switch (plan->config) {
         case 0: launch<Ig0>(ctx, p); break;
         case 1: launch<Ig1>(ctx, p); break;

@@ -323,6 +323,19 @@ int fc_conv_implicit_gemm(fc_context *ctx, const fc_igemm_plan *plan, const floa
                           const float *Wp_dev, const int32_t *table_dev,
                           const float *bias_dev, int relu, float *ws_dev, float *y_dev);
 
+/* The same layer for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): no counterpart in the reference.  The
+ * partial sums of a split reduction go to a static device array of FC_IGEMM_STATIC_WS_BYTES
+ * inside the library instead of a workspace of the caller's (each GPU the library runs on holds
+ * that array until the process ends); the call allocates nothing and is never bracketed by
+ * timing events.  A plan whose ws_bytes exceeds FC_IGEMM_STATIC_WS_BYTES is refused with
+ * FC_ERR_UNSUPPORTED.  All calls on one GPU share the array: calls that overlap in time on
+ * one GPU (two contexts, two streams) race; calls on one context are ordered and safe. */
+#define FC_IGEMM_STATIC_WS_BYTES (32 << 20)
+int fc_conv_implicit_gemm_static(fc_context *ctx, const fc_igemm_plan *plan, const float *x_dev,
+                                 const float *Wp_dev, const int32_t *table_dev,
+                                 const float *bias_dev, int relu, float *y_dev);
+
 /* ---- recorded launch sequences ----------------------------------------- */
 
 /* Records every launch made on the context between fc_graph_begin and fc_graph_end into a

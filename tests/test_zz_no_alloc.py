@@ -1,0 +1,71 @@
+"""fc_conv_implicit_gemm_static (split-reduction workspace in a static device array, no allocation)
+against fc_conv_implicit_gemm with a workspace of the caller's: same bits, on two calls in a row,
+the second with a smaller input; and against the fp64 oracle."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TOL_IM2COL = 1e-5
+
+
+def cshape(s):
+    import fastconv_amd as F
+    return F.ConvShape(*[getattr(s, n) for n, _ in F.ConvShape._fields_])
+
+
+def _both(L, shp, seed):
+    s = O.shape(*shp)
+    cs = cshape(s)
+    plan = L.igemm_plan(cs, L.igemm_default_config(cs))
+    x, w = O.make_inputs(s, seed=seed)
+    bias = O.rng_uniform(seed + 50, (s.K,))
+    mark = L.mark()
+    try:
+        dx, dw, db = L.upload(x), L.upload(w), L.upload(bias)
+        Wp, tab = L.alloc(plan.Wp_bytes), L.alloc(plan.table_bytes)
+        nout = s.N * s.K * plan.OH * plan.OW
+        y1, y2 = L.alloc(4 * nout), L.alloc(4 * nout)
+        ws = L.alloc(plan.ws_bytes) if plan.ws_bytes else None
+        L.igemm_pack_filter(plan, dw, Wp, tab)
+        L.fill_zero(y1, 4 * nout)
+        L.fill_zero(y2, 4 * nout)
+        L.conv_implicit_gemm(plan, dx, Wp, tab, y1, db, True, ws)
+        L.conv_implicit_gemm_static(plan, dx, Wp, tab, y2, db, True)
+        shape_out = (s.N, s.K, plan.OH, plan.OW)
+        a, b = L.download(y1, shape_out), L.download(y2, shape_out)
+    finally:
+        L.release(mark)
+    truth = np.maximum(O.naive_conv_f64(s, x, w, bias), 0.0)
+    return plan, a, b, truth
+
+
+def test_static_workspace_entry_point_matches_the_caller_workspace_one():
+    import fastconv_amd as F
+    from fastconv_amd import capi
+    L = F.load(0, 2 << 30)
+    try:
+        # a split reduction that nearly fills the static workspace, then a smaller one, then an unsplit layer
+        for shp, seed in [((1, 256, 56, 56, 256, 3, 3, 1, 1, 1), 1), ((1, 512, 14, 14, 512, 3, 3, 2, 2, 1), 2),
+                          ((1, 2048, 7, 7, 512, 1, 1, 1, 1, 0), 3), ((32, 64, 28, 28, 128, 3, 3, 1, 1, 1), 4)]:
+            print("static workspace", shp, flush=True)
+            plan, a, b, truth = _both(L, shp, seed)
+            if seed < 4:
+                assert plan.split_k > 1 and 0 < plan.ws_bytes <= capi.IGEMM_STATIC_WS_BYTES
+            else:
+                assert plan.split_k == 1
+            assert np.abs(a).max() > 0
+            assert np.array_equal(a, b), shp
+            assert O.max_rel_err(b, truth) <= TOL_IM2COL
+        # a layer whose partial sums do not fit is refused, and nothing is launched
+        big = cshape(O.shape(1, 256, 56, 56, 256))
+        plan = L.igemm_plan(big, 0)            # 128x128 tiles: few workgroups, many parts
+        assert plan.ws_bytes > capi.IGEMM_STATIC_WS_BYTES
+        buf = L.alloc(1 << 20)
+        with pytest.raises(F.FastConvError) as e:
+            L.conv_implicit_gemm_static(plan, buf, buf, buf, buf)
+        assert e.value.status == -6 and "static" in str(e.value)
+    finally:
+        L.close()
