@@ -5,15 +5,25 @@ A "step" is one forward pass of every conv layer of the workload (default: the
 13 3x3 conv layers of VGG-16 at batch 32, Winograd F(6x6,3x3), filter transform
 included) over synthetic inputs already resident in HBM.  Prints ONE JSON line:
 whole-job effective GFLOP/s (direct-convolution FLOP count / wall time), the
-roofline of the dominant kernel (the batched Winograd GEMM, timed with HIP
-events on the library's stream inside the timed region), and a CPU baseline (the
+roofline of the dominant kernel (timed with HIP events on the library's stream),
+a compact `secondary` list (the batch-1 stack, the ResNet-50 layers, the three
+im2col layers, each with the library's untuned choices) and a CPU baseline (the
 naive direct convolution on the host cores, on a bounded sample).
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--tune]
+
+Tile shape, pipeline and algorithm per layer are the library's own untuned
+choices (what the layer classes use without -tn tuning), so that a profiler run
+of this same command sees the same kernels; --tune searches them per layer
+first, as Tuning() of the layer classes does.  The stress workloads (batch 64
+and 128) always search, and report the staged ("ZC") and the blocked layer
+class side by side.
 """
 import argparse
+import ctypes
 import json
 import os
+import re
 import sys
 import time
 
@@ -24,21 +34,16 @@ sys.path.insert(0, ROOT)
 
 PEAK_MFMA_F32_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch of the GEMM kernel per layer (C, K, H) at batch 32: FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000
-# (factors from the plain copy kernel), from profiles/vgg16_b32_winograd_hbm_traffic_pmc.txt.  The counters need
-# their own rocprofv3 runs, so they are not re-measured by every bench run; `roofline.traffic` is their average
-# over the GEMM launches of a step.
-MEASURED_GEMM_TRAFFIC = {
-    32: {(128, 128, 112): 768.1e6, (128, 256, 56): 330.4e6, (256, 256, 56): 456.2e6, (256, 512, 28): 197.2e6,
-         (512, 512, 28): 289.7e6, (512, 512, 14): 155.1e6},
-}
+# Measured HBM bytes per launch of the GEMM kernels (FETCH_SIZE and WRITE_SIZE of rocprofv3 --pmc, scaled by what
+# the same counters read for a plain copy): a text summary under profiles/, one line per layer and tile shape.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemm_hbm_traffic_pmc.txt")
 
 # (C, K, H, repeats): 3x3, stride 1, pad 1
 VGG16 = [(3, 64, 224, 1), (64, 64, 224, 1), (64, 128, 112, 1), (128, 128, 112, 1), (128, 256, 56, 1),
          (256, 256, 56, 2), (256, 512, 28, 1), (512, 512, 28, 2), (512, 512, 14, 3)]
 RESNET50_3X3 = [(64, 64, 56, 3), (128, 128, 28, 4), (256, 256, 14, 6), (512, 512, 7, 3)]
 STRESS = [(256, 256, 56, 1), (512, 512, 28, 1), (512, 512, 14, 1)]
-# (C, K, H, kernel, stride, pad, repeats): the ResNet-50 bottleneck layers of BASELINE config 4
+# (C, K, H, kernel, stride, pad, repeats): the ResNet-50 bottleneck layers
 RESNET50 = [(3, 64, 224, 7, 2, 3, 1),
             (64, 64, 56, 1, 1, 0, 1), (64, 64, 56, 3, 1, 1, 3), (64, 256, 56, 1, 1, 0, 4), (256, 64, 56, 1, 1, 0, 2),
             (256, 128, 56, 1, 1, 0, 1), (128, 128, 56, 3, 2, 1, 1), (128, 128, 28, 3, 1, 1, 3),
@@ -58,36 +63,46 @@ WORKLOADS = {
     # name: (layers, batch, algorithm, description)
     "vgg16_b32": (_w(VGG16), 32, "winograd", "VGG-16 conv stack, 13 layers, 3x3 s1 p1, Winograd F(6,3), batch 32"),
     "vgg16_b1": (_w(VGG16), 1, "winograd", "VGG-16 conv stack, 13 layers, 3x3 s1 p1, Winograd F(6,3), batch 1"),
-    "vgg16_auto_b32": (_w(VGG16), 32, "auto", "VGG-16 conv stack, faster of Winograd / implicit GEMM per layer, batch 32"),
-    "vgg16_auto_b1": (_w(VGG16), 1, "auto", "VGG-16 conv stack, faster of Winograd / implicit GEMM per layer, batch 1"),
-    "resnet50_b32": (RESNET50, 32, "auto", "ResNet-50 conv layers (53 convs), auto algorithm per layer, batch 32"),
-    "resnet50_b1": (RESNET50, 1, "auto", "ResNet-50 conv layers (53 convs), auto algorithm per layer, batch 1"),
+    "vgg16_auto_b32": (_w(VGG16), 32, "auto", "VGG-16 conv stack, algorithm chosen per layer, batch 32"),
+    "vgg16_auto_b1": (_w(VGG16), 1, "auto", "VGG-16 conv stack, algorithm chosen per layer, batch 1"),
+    "resnet50_b32": (RESNET50, 32, "auto", "ResNet-50 conv layers (53 convs), algorithm chosen per layer, batch 32"),
+    "resnet50_b1": (RESNET50, 1, "auto", "ResNet-50 conv layers (53 convs), algorithm chosen per layer, batch 1"),
     "resnet50_3x3_b32": (_w(RESNET50_3X3), 32, "winograd", "ResNet-50 3x3 s1 convs, Winograd F(6,3), batch 32"),
     "resnet50_3x3_b1": (_w(RESNET50_3X3), 1, "winograd", "ResNet-50 3x3 s1 convs, Winograd F(6,3), batch 1"),
-    "im2col_abc_b1": (IM2COL_ABC, 1, "im2col", "BASELINE config 2: 3x3 256@56, 3x3 s2 128->256@56, 1x1 256->1024@14, batch 1"),
+    "im2col_abc_b1": (IM2COL_ABC, 1, "im2col", "3x3 256@56, 3x3 s2 128->256@56, 1x1 256->1024@14 through the implicit GEMM, batch 1"),
     "cfg1": (_w([(64, 64, 56, 1)]), 1, "winograd", "single 3x3 conv 64->64 @56, batch 1"),
     "conv64_224_b32": (_w([(64, 64, 224, 1)]), 32, "winograd", "single 3x3 conv 64->64 @224, batch 32 (VGG-16 layer 2)"),
-    "stress_b64": (_w(STRESS), 64, "winograd", "VGG-16 256@56, 512@28, 512@14, batch 64"),
-    "stress_b128": (_w(STRESS), 128, "winograd", "VGG-16 256@56, 512@28, 512@14, batch 128"),
+    "conv256_56_b32": (_w([(256, 256, 56, 1)]), 32, "winograd", "single 3x3 conv 256->256 @56, batch 32 (VGG-16 layers 6-7)"),
+    "conv512_28_b32": (_w([(512, 512, 28, 1)]), 32, "winograd", "single 3x3 conv 512->512 @28, batch 32 (VGG-16 layers 9-10)"),
+    "stress_b64": (_w(STRESS), 64, "winograd", "VGG-16 256@56, 512@28, 512@14 at batch 64: staged (ZC) against blocked Winograd, tile shapes searched"),
+    "stress_b128": (_w(STRESS), 128, "winograd", "VGG-16 256@56, 512@28, 512@14 at batch 128: staged (ZC) against blocked Winograd, tile shapes searched"),
 }
+SECONDARY = ("vgg16_b1", "resnet50_b32", "im2col_abc_b1")
 
-ST_KT, ST_IT, ST_GEMM, ST_OT = 0, 1, 2, 3
+ST_KT, ST_IT, ST_GEMM, ST_OT, ST_IGEMM, ST_FUSED, ST_ONEPASS = 0, 1, 2, 3, 4, 6, 7
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def _offset(ptr, nbytes):
+    return ctypes.c_void_p(ptr.value + nbytes)
+
+
 class Layer:
     """One conv layer with its buffers resident on the device."""
 
-    def __init__(self, L, F, N, spec, rng):
+    def __init__(self, L, F, N, spec, index):
+        from fastconv_amd import capi
         C, K, H, ks, st, pad, repeats = spec
         self.N, self.C, self.K, self.H, self.ks, self.st, self.pad, self.repeats = N, C, K, H, ks, st, pad, repeats
+        self.F = F
         self.shape = F.ConvShape(N, C, H, H, K, ks, ks, st, st, pad, pad, pad, pad)
         self.OH = self.shape.out_hw()[0]
-        x = rng.random((N, C, H, H), dtype=np.float32) * 2.0 - 1.0
-        w = (rng.standard_normal((K, C, ks, ks), dtype=np.float32) * np.float32(np.sqrt(2.0 / (ks * ks * C))))
+        # the workload's inputs: uniform [-1, 1), He-normal weights, seeded per layer
+        x = capi.host_uniform(2 * index + 1, (N, C, H, H))
+        w = capi.host_normal(2 * index + 2, (K, C, ks, ks), float(np.sqrt(2.0 / (ks * ks * C))))
         self.x, self.w = L.upload(x), L.upload(w)
         self.y = L.alloc(4 * N * K * self.OH * self.OH)
         self.flops = self.shape.flops()
@@ -95,9 +110,12 @@ class Layer:
         self.plan = None              # Winograd plan
         self.U = None
         self.pipe = "staged"          # Winograd pipeline: staged, fused (GEMM + output transform) or onepass
+        self.img_block = N            # fused pipeline: images per block (the blocked layer class)
+        self.block_plans = None
         self.oplan = self.U2 = None   # single-kernel path: its plan and its filter layout
         self.iplan = self.Wp = self.table = self.ws = None   # implicit GEMM
         self.wino_ok = ks == 3 and st == 1
+        self.candidates = None
 
     @property
     def fused(self):
@@ -108,6 +126,17 @@ class Layer:
             self.oplan = L.wino_onepass_plan(self.shape)
             self.U2 = L.alloc(self.oplan.U_bytes)
             L.wino_onepass_filter_transform(self.oplan, self.w, self.U2)
+
+    def set_blocks(self, L, cfg, img_block):
+        """Plans for the blocked class: the batch cut into blocks of img_block images."""
+        self.img_block = img_block
+        self.block_plans = None
+        if img_block < self.N:
+            def plan_for(n):
+                s = self.F.ConvShape(n, self.C, self.H, self.H, self.K, 3, 3, 1, 1, 1, 1, 1, 1)
+                return L.wino_plan(s, cfg)
+            tail = self.N % img_block
+            self.block_plans = (plan_for(img_block), plan_for(tail) if tail else None)
 
     def name(self):
         tag = "" if (self.ks, self.st) == (3, 1) else " %dx%d/s%d" % (self.ks, self.ks, self.st)
@@ -131,14 +160,23 @@ class Layer:
 
 
 def forward(L, lay, V, M, filter_ready=False):
-    """One layer pass: implicit GEMM, or Winograd staged (four kernels) or fused (GEMM + output
-    transform in one kernel)."""
+    """One layer pass: implicit GEMM, or Winograd staged (the ZC class: filter + input transform,
+    GEMM, output transform), fused (the blocked class: GEMM + output transform in one kernel, per
+    block of images) or onepass (the blocked class taken to its end: one kernel)."""
     if lay.algo == "im2col":
         L.conv_implicit_gemm(lay.iplan, lay.x, lay.Wp, lay.table, lay.y, ws=lay.ws)
     elif lay.pipe == "onepass":
         L.wino_forward_onepass(lay.oplan, lay.x, lay.w, lay.U2, lay.y, filter_ready=filter_ready)
     elif lay.fused:
-        L.wino_forward_fused(lay.plan, lay.x, lay.w, lay.U, V, lay.y, filter_ready=filter_ready)
+        if lay.block_plans is None:
+            L.wino_forward_fused(lay.plan, lay.x, lay.w, lay.U, V, lay.y, filter_ready=filter_ready)
+        else:
+            in_img, out_img = 4 * lay.C * lay.H * lay.H, 4 * lay.K * lay.OH * lay.OH
+            full, tail = lay.block_plans
+            for n0 in range(0, lay.N, lay.img_block):
+                p = full if n0 + lay.img_block <= lay.N else tail
+                L.wino_forward_fused(p, _offset(lay.x, n0 * in_img), lay.w, lay.U, V, _offset(lay.y, n0 * out_img),
+                                     filter_ready=filter_ready or n0 > 0)
     else:
         L.wino_forward(lay.plan, lay.x, lay.w, lay.U, V, M, lay.y, filter_ready=filter_ready)
 
@@ -153,10 +191,21 @@ def _time(L, fn, iters):
     return (time.perf_counter() - t0) / iters * 1e3
 
 
-def tune_layer(L, lay, V, M, scratch_bytes, iters=3):
-    """Pick the GEMM tile shape and pipeline with the shortest whole-layer forward."""
-    best = (None, "staged", 1e30)
+def tune_layer(L, lay, V, M, scratch_bytes, iters=3, full_search=False):
+    """Whole-layer forward time of every candidate: tile shape x pipeline (x images per block for the
+    blocked class when full_search).  Returns the best as (cfg, pipe, ms, img_block) and keeps the table
+    of the best candidate per layer class in lay.candidates."""
+    best = (None, "staged", 1e30, lay.N)
+    per_class = {}
     lay.algo = "winograd"
+
+    def note(cls, cfg, pipe, ms, ib):
+        nonlocal best
+        if ms < best[2]:
+            best = (cfg, pipe, ms, ib)
+        if cls not in per_class or ms < per_class[cls]["ms"]:
+            per_class[cls] = {"cfg": cfg, "pipe": pipe, "ms": ms, "img_block": ib}
+
     for cfg in L.wino_configs():
         plan = L.wino_plan(lay.shape, cfg.id)
         if plan.V_bytes > scratch_bytes[0] or plan.M_bytes > scratch_bytes[1]:
@@ -166,19 +215,29 @@ def tune_layer(L, lay, V, M, scratch_bytes, iters=3):
         lay.plan = plan
         mark = L.mark()
         lay.U = L.alloc(plan.U_bytes)
+        lay.pipe = "staged"
+        lay.set_blocks(L, cfg.id, lay.N)
+        note("zc", cfg.id, "staged", _time(L, lambda: forward(L, lay, V, M), iters), lay.N)
         # the fused kernel has one tile shape of its own; the plan only fixes the padding it reads
-        for pipe in (("staged", "fused") if lay.C * lay.K <= 16384 else ("staged",)):
-            lay.pipe = pipe
-            ms = _time(L, lambda: forward(L, lay, V, M), iters)
-            if ms < best[2]:
-                best = (cfg.id, pipe, ms)
+        if full_search or lay.C * lay.K <= 16384:
+            lay.pipe = "fused"
+            blocks = [lay.N] + ([lay.N // 2, lay.N // 4] if full_search and cfg.id in (0, 3) and lay.N >= 4 else [])
+            for ib in blocks:
+                lay.set_blocks(L, cfg.id, ib)
+                note("blocked", cfg.id, "fused", _time(L, lambda: forward(L, lay, V, M), iters), ib)
+            lay.set_blocks(L, cfg.id, lay.N)
         L.release(mark)
-    if lay.C <= 128:      # the whole layer in one kernel: no tile shape to choose
-        lay.setup_onepass(L)
-        lay.pipe = "onepass"
-        ms = _time(L, lambda: forward(L, lay, V, M), iters)
-        if ms < best[2]:
-            best = (best[0], "onepass", ms)
+    if full_search or lay.C <= 128:      # the whole layer in one kernel: no tile shape to choose
+        try:
+            lay.setup_onepass(L)
+        except lay.F.FastConvError:
+            pass
+        else:
+            lay.pipe = "onepass"
+            note("blocked", None, "onepass", _time(L, lambda: forward(L, lay, V, M), iters), lay.N)
+    if best[0] is None:      # the single-kernel engine won outright: the plan below still needs a tile shape
+        best = (L.wino_default_config(lay.shape),) + best[1:]
+    lay.candidates = per_class
     return best
 
 
@@ -195,9 +254,10 @@ def tune_im2col(L, lay, iters=3):
     return best
 
 
-def cpu_baseline(target_seconds=12.0):
+def cpu_baseline(target_seconds=3.0):
     """Naive direct convolution (the oracle's restatement of the reference's
-    ConvNaiveLayer, OpenMP over images x output channels) on the VGG-16 stack."""
+    ConvNaiveLayer, OpenMP over images x output channels) on the VGG-16 stack,
+    on a sample of about target_seconds of host time."""
     from oracle import oracle as O
     cores = O.lib().fco_num_threads()
 
@@ -214,13 +274,13 @@ def cpu_baseline(target_seconds=12.0):
         return total_flops, total_s
 
     fl, s1 = run(1)
-    batch = int(max(1, min(32, target_seconds // max(s1, 1e-3))))
+    batch = int(max(1, min(32, (target_seconds - s1) // max(s1, 1e-3))))
     if batch > 1:
         fl, s1 = run(batch)
     return {"value": round(fl / s1 / 1e9, 2), "unit": "GFLOP/s", "cores": cores, "kind": "port",
             "sample": "naive direct conv (restatement of the reference's ConvNaiveLayer; the reference's NEON "
-                      "kernels do not build on this x86 host), VGG-16 13-layer conv stack at batch %d, %.1f s"
-                      % (batch, s1)}
+                      "kernels do not build on this x86 host), VGG-16 13-layer conv stack at batch %d, %.1f s "
+                      "of host time (repeated layers timed once)" % (batch, s1)}
 
 
 def copy_probe(mib):
@@ -244,45 +304,27 @@ def copy_probe(mib):
     L.close()
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="vgg16_b32", choices=sorted(WORKLOADS))
-    ap.add_argument("--no-tune", action="store_true", help="use the built-in default tile shape per layer")
-    ap.add_argument("--offline-filter", action="store_true",
-                    help="transform the filters once outside the timed region")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--stage-events", default="auto", choices=["auto", "all", "gemm", "none"],
-                    help="which kernels are bracketed by events inside the timed region.  An event pair costs "
-                         "5-8 us per launch: 'gemm' brackets the dominant kernel only (the other kernels are "
-                         "bracketed in a few extra untimed steps), 'none' brackets nothing in the timed region "
-                         "(everything comes from the untimed steps).  'auto' (default) is 'gemm' while the "
-                         "brackets cost under 2 %% of a step (VGG-16 at batch 32: 9 launches in 3.5 ms), else "
-                         "'none' (ResNet-50: 53 launches, 15 %% of the step; batch-1 stacks)")
-    ap.add_argument("--pipeline", default="auto", choices=["auto", "staged", "fused", "onepass"],
-                    help="Winograd pipeline per layer: four staged kernels, GEMM + output transform fused, or "
-                         "whichever is faster for the layer (auto)")
-    ap.add_argument("--graph", action="store_true",
-                    help="record one step as a HIP graph and time replays of it (per-launch events are off; "
-                         "the default times the per-layer calls the reference's driver makes)")
-    ap.add_argument("--timed-only", action="store_true",
-                    help="no per-layer detail pass after the timed region (every launch of the process is then a "
-                         "warm-up or timed step: what a kernel trace of this command averages over)")
-    ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
-                    help="only run the plain copy kernel over MIB mebibytes (scale for the HBM traffic counters)")
-    args = ap.parse_args()
-    if args.copy_probe:
-        return copy_probe(args.copy_probe)
-    if args.gpus != 1:
-        print("bench.py: this build runs on one GPU only (the layers shard by batch with no exchange step: "
-              "each GPU would hold the transformed filter and its share of the images); run with --gpus 1", file=sys.stderr)
-        sys.exit(2)
+def measured_traffic():
+    """{(kernel, N, C, K, H, ks, st, 'BMxBNxBK'): bytes per launch} parsed from the committed rocprofv3 counter
+    summary; empty when the file is absent (`traffic` is then null)."""
+    out = {}
+    if not os.path.exists(TRAFFIC_PROFILE):
+        return out
+    pat = re.compile(r"^traffic kernel=(\w+) N=(\d+) C=(\d+) K=(\d+) H=(\d+) ks=(\d+) st=(\d+) tile=(\w+) "
+                     r".*measured_bytes=(\d+)")
+    for line in open(TRAFFIC_PROFILE):
+        m = pat.match(line.strip())
+        if m:
+            out[(m.group(1),) + tuple(int(m.group(i)) for i in range(2, 8)) + (m.group(8),)] = int(m.group(9))
+    return out
 
+
+def run_workload(name, steps, warmup, o, detail=True):
+    """Builds the layers of one workload on the device, times `steps` steps and returns the result fields."""
     import fastconv_amd as F
-    layers_def, N, algo, desc = WORKLOADS[args.workload]
-    rng = np.random.default_rng(0)
+    layers_def, N, algo, desc = WORKLOADS[name]
+    stress = name.startswith("stress")
+    tune = o.tune or stress
 
     # arena: activations + filters + U / packed filter per layer, one shared V and M (largest layer)
     act = sum(4 * N * (C * H * H + K * (H // st + 1) ** 2) for (C, K, H, ks, st, pad, _) in layers_def)
@@ -296,51 +338,47 @@ def main():
     pool = int(act + vmax + mmax + umax + imax + (512 << 20))
     L = F.load(0, pool)
     info = L.device_info()
-    log("device:", info)
+    log("workload %s on %s" % (name, info["arch"]))
     V, M = L.alloc(vmax), L.alloc(mmax)
-    layers = [Layer(L, F, N, spec, rng) for spec in layers_def]
+    layers = [Layer(L, F, N, spec, i) for i, spec in enumerate(layers_def)]
 
-    # tile shape per layer
+    # algorithm, pipeline and tile shape per layer
     for lay in layers:
         want_wino = lay.wino_ok and algo in ("winograd", "auto")
         want_im2col = algo == "im2col" or not lay.wino_ok or algo == "auto"
         if algo == "winograd" and not lay.wino_ok:
-            raise SystemExit("workload %s: Winograd needs 3x3 stride 1" % args.workload)
+            raise SystemExit("workload %s: Winograd needs 3x3 stride 1" % name)
         wres = ires = None
         if want_wino:
-            if args.no_tune:      # the library's untuned choices
+            if not tune:      # the library's untuned choices
                 wres = (L.wino_default_config(lay.shape),
                         "onepass" if L.wino_prefer_onepass(lay.shape) else
-                        "fused" if L.wino_prefer_fused(lay.shape) else "staged", 0.0)
+                        "fused" if L.wino_prefer_fused(lay.shape) else "staged", 0.0, N)
             else:
-                wres = tune_layer(L, lay, V, M, (vmax, mmax))
+                wres = tune_layer(L, lay, V, M, (vmax, mmax), full_search=stress)
         if want_im2col:
-            if args.no_tune:
-                ires = (L.igemm_default_config(lay.shape), 0.0)
-            else:
-                ires = tune_im2col(L, lay)
+            ires = (L.igemm_default_config(lay.shape), 0.0) if not tune else tune_im2col(L, lay)
         if wres and ires:
-            if args.no_tune:      # the driver's rule for -a auto: Winograd unless few channels or few tiles
-                T = N * ((lay.H + 5) // 6) ** 2
-                use_w = not (lay.C < 16 or (T < 64 and lay.C * lay.K >= 128 * 128))
-            else:
-                use_w = wres[2] <= ires[1]
+            # -a auto: the library's rule, or the measured winner when both were timed
+            use_w = L.prefer_winograd(lay.shape) if not tune else wres[2] <= ires[1]
+            lay.auto_times = None if not tune else {"winograd_ms": round(wres[2], 4), "im2col_ms": round(ires[1], 4),
+                                                    "rule_says": "winograd" if L.prefer_winograd(lay.shape) else "im2col"}
         else:
             use_w = wres is not None
         if use_w:
-            cfg, pipe, ms = wres
-            if args.pipeline != "auto":
-                pipe = args.pipeline
+            cfg, pipe, ms, ib = wres
+            if o.pipeline != "auto":
+                pipe = o.pipeline
             lay.algo, lay.pipe = "winograd", pipe
             if pipe == "onepass":
                 lay.setup_onepass(L)
             lay.plan = L.wino_plan(lay.shape, cfg)
             lay.U = L.alloc(lay.plan.U_bytes)
+            lay.set_blocks(L, cfg, ib if pipe == "fused" else N)
             L.wino_filter_transform(lay.plan, lay.w, lay.U)
             g = L.wino_configs()[cfg]
             log("layer %s: winograd %s, tile %dx%dx%d (cfg %d) %.3f ms%s"
-                % (lay.name(), pipe, g.bm, g.bn, g.bk, cfg, ms,
-                   " (im2col %.3f ms)" % ires[1] if ires else ""))
+                % (lay.name(), pipe, g.bm, g.bn, g.bk, cfg, ms, " (im2col %.3f ms)" % ires[1] if ires else ""))
         else:
             cfg, ms = ires
             lay.algo = "im2col"
@@ -351,18 +389,19 @@ def main():
                    " (winograd %.3f ms)" % wres[2] if wres else ""))
     L.sync()
 
-    filter_ready = args.offline_filter
+    filter_ready = o.offline_filter
 
     def step():
         for lay in layers:
             for _ in range(lay.repeats):
                 forward(L, lay, V, M, filter_ready)
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     L.sync()
 
-    if args.stage_events == "auto":
+    stage_events = o.stage_events
+    if stage_events == "auto":
         # one more untimed step for a rough step time: brackets stay inside the timed region while
         # their own cost (about 6 us per bracketed launch) is under 2 % of the step
         t0 = time.perf_counter()
@@ -370,10 +409,10 @@ def main():
         L.sync()
         rough_us = (time.perf_counter() - t0) * 1e6
         bracketed = sum(l.repeats for l in layers if l.algo == "im2col" or l.pipe == "staged")
-        args.stage_events = "gemm" if 6.0 * bracketed <= 0.02 * rough_us else "none"
-    mask = {"all": 0xdf, "gemm": (1 << ST_GEMM) | (1 << 4), "none": 0}[args.stage_events]
+        stage_events = "gemm" if 6.0 * bracketed <= 0.02 * rough_us else "none"
+    mask = {"all": 0xdf, "gemm": (1 << ST_GEMM) | (1 << ST_IGEMM), "none": 0}[stage_events]
     timed_step = step
-    if args.graph:
+    if o.graph:
         mask = 0
         L.graph_begin()
         step()
@@ -384,39 +423,39 @@ def main():
     L.timing(mask)
     L.timing_reset()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         timed_step()
     L.sync()
     elapsed = time.perf_counter() - t0
     stage = [L.stage_time(i) for i in range(4)]
-    fused_stage = L.stage_time(6)
-    onepass_stage = L.stage_time(7)
-    igemm_stage = L.stage_time(4)
+    fused_stage = L.stage_time(ST_FUSED)
+    onepass_stage = L.stage_time(ST_ONEPASS)
+    igemm_stage = L.stage_time(ST_IGEMM)
     L.timing(0)
-    if args.stage_events != "all" and not args.timed_only:
+    if stage_events != "all" and not o.timed_only:
         # the other kernels: the same steps again, untimed, every kernel bracketed
         L.timing(0xdf)
         L.timing_reset()
-        for _ in range(min(args.steps, 5)):
+        for _ in range(min(steps, 5)):
             step()
         L.sync()
-        detail = [L.stage_time(i) for i in range(4)]
+        detail_t = [L.stage_time(i) for i in range(4)]
         for i in (ST_KT, ST_IT, ST_OT):
-            stage[i] = detail[i]
-        fused_stage = L.stage_time(6)
-        onepass_stage = L.stage_time(7)
-        if args.stage_events == "none" or args.graph:
-            stage[ST_GEMM] = detail[ST_GEMM]
-            igemm_stage = L.stage_time(4)
+            stage[i] = detail_t[i]
+        fused_stage = L.stage_time(ST_FUSED)
+        onepass_stage = L.stage_time(ST_ONEPASS)
+        if stage_events == "none" or o.graph:
+            stage[ST_GEMM] = detail_t[ST_GEMM]
+            igemm_stage = L.stage_time(ST_IGEMM)
         L.timing(0)
 
-    ms_per_step = elapsed / args.steps * 1e3
+    ms_per_step = elapsed / steps * 1e3
     # shader clock under this workload: the same steps once more, untimed, beside the library's
     # clock probe (the published MFMA peak is quoted at the maximum clock; power management runs
     # the shaders slower under fp32 MFMA load with real data)
     shader_clock = None
-    if not args.timed_only:
-        n_probe = max(3, min(args.steps, 10))
+    if detail and not o.timed_only:
+        n_probe = max(3, min(steps, 10))
         samples = 64
         sample_us = int(min(100000, max(20, ms_per_step * 1e3 * n_probe / samples)))
         step()
@@ -426,25 +465,32 @@ def main():
             step()
         L.sync()
         mhz = L.clock_probe_end()
-        shader_clock = {"nominal_mhz": None, "mean_mhz": round(sum(mhz) / len(mhz), 1), "min_mhz": round(min(mhz), 1),
-                        "max_mhz": round(max(mhz), 1), "samples": len(mhz), "sample_us": sample_us,
-                        "over": "%d more steps of the same workload, untimed" % n_probe}
+        shader_clock = {"nominal_mhz": info["clock_mhz"], "mean_mhz": round(sum(mhz) / len(mhz), 1),
+                        "min_mhz": round(min(mhz), 1), "max_mhz": round(max(mhz), 1), "samples": len(mhz),
+                        "sample_us": sample_us, "over": "%d more steps of the same workload, untimed" % n_probe}
     step_flops = sum(l.flops * l.repeats for l in layers)
     value = step_flops / (ms_per_step * 1e-3) / 1e9
 
     # dominant kernel: the batched GEMM. achieved = algorithmic flops of all its launches / their event time
+    traffic = measured_traffic()
     wino = [l for l in layers if l.algo == "winograd"]
     staged = [l for l in wino if l.pipe == "staged"]
     gemm_flops_step = sum(l.algorithmic()["gemm_flops"] * l.repeats for l in staged)
     launches_step = max(1, sum(l.repeats for l in staged))
     roofline = {"kernel": "wino_gemm_kernel", "bound": "mfma", "achieved": None, "peak": PEAK_MFMA_F32_TFLOPS,
                 "unit": "TFLOP/s", "frac": None, "traffic": None}
+
+    def tile_name(g):
+        return "%dx%dx%d" % (g.bm, g.bn, g.bk)
+
     if stage[ST_GEMM][1] > 0:
         gemm_ms, gemm_cnt = stage[ST_GEMM]
         ach = gemm_flops_step * (gemm_cnt / launches_step) / (gemm_ms * 1e-3) / 1e12
-        known = MEASURED_GEMM_TRAFFIC.get(N, {})
-        if staged and all((l.C, l.K, l.H) in known for l in staged):
-            roofline["traffic"] = round(sum(known[(l.C, l.K, l.H)] * l.repeats for l in staged) / launches_step)
+        keys = [("wino_gemm_kernel", N, l.C, l.K, l.H, 3, 1, tile_name(L.wino_configs()[l.plan.gemm_config]))
+                for l in staged]
+        if staged and all(k in traffic for k in keys):
+            roofline["traffic"] = round(sum(traffic[k] * l.repeats for k, l in zip(keys, staged)) / launches_step)
+            roofline["traffic_source"] = os.path.relpath(TRAFFIC_PROFILE, ROOT)
         roofline["algorithmic_bytes_per_launch_avg"] = round(
             sum(256.0 * (l.K * l.C + l.C * l.plan.T + l.K * l.plan.T) * l.repeats for l in staged) / launches_step)
         roofline.update(achieved=round(ach, 2), frac=round(ach / PEAK_MFMA_F32_TFLOPS, 4),
@@ -457,8 +503,8 @@ def main():
     transforms = {}
     # online filter transforms of the staged and fused pipelines ride in the input transform's launch
     merged = [l for l in wino if l.pipe != "onepass"] if not filter_ready else []
-    for name, idx, key in (("input_transform", ST_IT, "it_bytes"), ("output_transform", ST_OT, "ot_bytes"),
-                           ("filter_transform", ST_KT, "kt_bytes")):
+    for tname, idx, key in (("input_transform", ST_IT, "it_bytes"), ("output_transform", ST_OT, "ot_bytes"),
+                            ("filter_transform", ST_KT, "kt_bytes")):
         ms, cnt = stage[idx]
         if cnt > 0:
             if idx == ST_OT:
@@ -467,23 +513,24 @@ def main():
                 who = [l for l in wino if l.pipe != "onepass"]
             else:
                 who = [l for l in wino if l not in merged]
-            per_step = max(1, sum(l.repeats for l in who))
+            per_step = max(1, sum(l.repeats * (1 if idx != ST_IT or l.block_plans is None
+                                               else -(-l.N // l.img_block)) for l in who))
             b = sum(l.algorithmic()[key] * l.repeats for l in who)
             if idx == ST_IT:
                 b += sum(l.algorithmic()["kt_bytes"] * l.repeats for l in merged)
             b *= cnt / per_step
             gbs = b / (ms * 1e-3) / 1e9
-            transforms[name] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                "frac": round(gbs / PEAK_HBM_GBS, 4), "launches": cnt}
+            transforms[tname] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                 "frac": round(gbs / PEAK_HBM_GBS, 4), "launches": cnt}
             if idx == ST_IT and merged:
-                transforms[name]["includes"] = "filter transform (same launch)"
+                transforms[tname]["includes"] = "filter transform (same launch)"
 
     if fused_stage[1] > 0:
         fl = [l for l in wino if l.fused]
-        per_step = sum(l.repeats for l in fl)
         fbytes = sum((256.0 * (l.K * l.C + l.C * l.plan.T) + 4.0 * l.N * l.K * l.H * l.H) * l.repeats for l in fl)
         fflops = sum(l.algorithmic()["gemm_flops"] * l.repeats for l in fl)
-        k = fused_stage[1] / per_step
+        per_step_launches = sum(l.repeats * (1 if l.block_plans is None else -(-l.N // l.img_block)) for l in fl)
+        k = fused_stage[1] / per_step_launches        # steps the events cover
         transforms["fused_gemm_output"] = {
             "bound": "hbm", "achieved": round(fbytes * k / (fused_stage[0] * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
             "unit": "GB/s", "frac": round(fbytes * k / (fused_stage[0] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
@@ -501,7 +548,8 @@ def main():
             "bound": "mfma", "achieved": round(oflops * k / (onepass_stage[0] * 1e-3) / 1e12, 2),
             "peak": PEAK_MFMA_F32_TFLOPS, "unit": "TFLOP/s",
             "frac": round(oflops * k / (onepass_stage[0] * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 4),
-            "launches": onepass_stage[1], "hbm_gbs": round(gbs, 1)}
+            "launches": onepass_stage[1], "avg_launch_ms": round(onepass_stage[0] / onepass_stage[1], 5),
+            "hbm_gbs": round(gbs, 1)}
 
     if igemm_stage[1] > 0:
         il = [l for l in layers if l.algo == "im2col"]
@@ -515,7 +563,13 @@ def main():
     # ResNet-50 workloads, the staged Winograd GEMM in the VGG-16 ones
     if igemm_stage[1] > 0 and (not staged or igemm_stage[0] > stage[ST_GEMM][0]):
         wino_gemm_line = roofline if staged and stage[ST_GEMM][1] > 0 else None
-        roofline = dict(transforms["implicit_gemm"], kernel="igemm_conv_kernel", traffic=None,
+        il = [l for l in layers if l.algo == "im2col"]
+        keys = [("igemm_conv_kernel", N, l.C, l.K, l.H, l.ks, l.st, tile_name(L.igemm_configs()[l.iplan.config]))
+                for l in il]
+        tr = None
+        if all(k in traffic for k in keys):
+            tr = round(sum(traffic[k] * l.repeats for k, l in zip(keys, il)) / sum(l.repeats for l in il))
+        roofline = dict(transforms["implicit_gemm"], kernel="igemm_conv_kernel", traffic=tr,
                         avg_launch_ms=round(igemm_stage[0] / igemm_stage[1], 5))
         if shader_clock:
             at_clock = info["compute_units"] * 256 * shader_clock["mean_mhz"] * 1e6 / 1e12
@@ -523,10 +577,12 @@ def main():
                             frac_at_measured_clock=round(roofline["achieved"] / at_clock, 4))
         if wino_gemm_line:
             transforms["wino_gemm"] = wino_gemm_line
+    elif not staged and onepass_stage[1] > 0:
+        roofline = dict(transforms["single_kernel_conv"], kernel="wino_onepass_kernel", traffic=None)
 
     # yardstick for the HBM-bound kernels: the library's plain copy kernel (16 bytes per lane) over the
     # V and M scratch, outside the timed region
-    if not args.timed_only:
+    if detail and not o.timed_only:
         nb = int(min(vmax, mmax, 1 << 30)) // 256 * 256
         if nb >= (64 << 20):
             L.device_copy(M, V, nb)
@@ -540,30 +596,66 @@ def main():
                                          "frac": round(gbs / PEAK_HBM_GBS, 4), "bytes": 2 * nb,
                                          "note": "read + write of a plain copy: what streaming kernels reach on this box"}
 
+    def class_detail(lay, cand):
+        """Time and GEMM-stage MFMA rate of one layer class's best candidate (events around every kernel)."""
+        cfg = cand["cfg"] if cand["cfg"] is not None else L.wino_default_config(lay.shape)
+        mark = L.mark()
+        lay.pipe, lay.plan = cand["pipe"], L.wino_plan(lay.shape, cfg)
+        lay.U = L.alloc(lay.plan.U_bytes)
+        lay.set_blocks(L, cfg, cand["img_block"] if cand["pipe"] == "fused" else lay.N)
+        L.timing(0xdf)
+        L.timing_reset()
+        forward(L, lay, V, M)
+        L.sync()
+        L.timing_reset()
+        reps = 5
+        for _ in range(reps):
+            forward(L, lay, V, M)
+        L.sync()
+        st = {i: L.stage_time(i)[0] / reps for i in (ST_KT, ST_IT, ST_GEMM, ST_OT, ST_FUSED, ST_ONEPASS)}
+        L.timing(0)
+        L.release(mark)
+        gemm_ms = st[ST_GEMM] + st[ST_FUSED] + st[ST_ONEPASS]
+        g = L.wino_configs()[cfg]
+        gf = lay.algorithmic()["gemm_flops"]
+        row = {"ms": round(cand["ms"], 4), "gflops": round(lay.flops / (cand["ms"] * 1e-3) / 1e9, 1),
+               "gemm_kernel_ms": round(gemm_ms, 4), "gemm_tflops": round(gf / (gemm_ms * 1e-3) / 1e12, 2),
+               "gemm_frac_mfma": round(gf / (gemm_ms * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 3)}
+        if cand["pipe"] == "staged":
+            row.update(engine="four staged kernels, whole-layer U/V/M", tile=tile_name(g), waves="%dx%d" % (g.waves_m, g.waves_n),
+                       input_tran_ms=round(st[ST_IT], 4), output_tran_ms=round(st[ST_OT], 4))
+        elif cand["pipe"] == "fused":
+            row.update(engine="GEMM + output transform in one kernel, no M buffer", tile="32x32x2 per wavefront, 8 wavefronts x 8 frequencies",
+                       padding_of="%s plan" % tile_name(g), images_per_block=cand["img_block"],
+                       input_tran_ms=round(st[ST_IT], 4))
+        else:
+            row.update(engine="single kernel (no V, no M)", tile="64 output channels x 16 tiles x 4 channels per chunk",
+                       images_per_block=lay.N)
+        return row
+
     # per-layer detail, outside the timed region
     per_layer = []
     L.timing(0xdf)
-    for lay in ([] if args.timed_only else layers):
+    for lay in ([] if (o.timed_only or not detail) else layers):
         L.timing_reset()
         reps = 5
         for _ in range(reps):
             forward(L, lay, V, M)
         L.sync()
         g = (L.igemm_configs()[lay.iplan.config] if lay.algo == "im2col" else L.wino_configs()[lay.plan.gemm_config])
-        row = {"layer": lay.name(), "batch": N, "repeats": lay.repeats, "algorithm": lay.algo,
-               "tile": "%dx%dx%d" % (g.bm, g.bn, g.bk)}
+        row = {"layer": lay.name(), "batch": N, "repeats": lay.repeats, "algorithm": lay.algo, "tile": tile_name(g)}
         if lay.algo == "im2col":
-            ms = L.stage_time(4)[0] / reps
+            ms = L.stage_time(ST_IGEMM)[0] / reps
             row.update(ms=round(ms, 4), gflops=round(lay.flops / (ms * 1e-3) / 1e9, 1), split_k=lay.iplan.split_k,
                        gemm_tflops=round(lay.flops / (ms * 1e-3) / 1e12, 2),
                        gemm_frac_mfma=round(lay.flops / (ms * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 3))
         else:
             st = [L.stage_time(i)[0] / reps for i in range(4)]
             if lay.fused:      # one kernel does the GEMM and the output transform: listed under gemm
-                st[ST_GEMM] = L.stage_time(6)[0] / reps
+                st[ST_GEMM] = L.stage_time(ST_FUSED)[0] / reps
                 st[ST_OT] = 0.0
             if lay.pipe == "onepass":      # one kernel does everything but the filter transform: listed under gemm
-                st[ST_GEMM] = L.stage_time(7)[0] / reps
+                st[ST_GEMM] = L.stage_time(ST_ONEPASS)[0] / reps
                 st[ST_IT] = st[ST_OT] = 0.0
             total = sum(st)
             a = lay.algorithmic()
@@ -577,33 +669,104 @@ def main():
                 "output_tran_gbs": round(a["ot_bytes"] / (st[ST_OT] * 1e-3) / 1e9, 0) if st[ST_OT] else None,
                 "stage_ms": {"kernel_tran": round(st[ST_KT], 4), "input_tran": round(st[ST_IT], 4),
                              "gemm": round(st[ST_GEMM], 4), "output_tran": round(st[ST_OT], 4)}})
+        if getattr(lay, "auto_times", None):
+            row["auto"] = lay.auto_times
         per_layer.append(row)
     L.timing(0)
+    if stress and detail:
+        # the two layer classes side by side: best candidate of each, with the parameters it chose
+        saved = [(l.pipe, l.plan, l.U, l.img_block, l.block_plans) for l in layers]
+        for lay, row in zip(layers, per_layer):
+            cands = lay.candidates or {}
+            if "zc" in cands:
+                row["zc_class"] = class_detail(lay, cands["zc"])
+            if "blocked" in cands:
+                row["blocked_class"] = class_detail(lay, cands["blocked"])
+            if "zc" in cands and "blocked" in cands:
+                row["faster_class"] = "zc" if cands["zc"]["ms"] <= cands["blocked"]["ms"] else "blocked"
+        for lay, (pipe, plan, U, ib, bp) in zip(layers, saved):
+            lay.pipe, lay.plan, lay.U, lay.img_block, lay.block_plans = pipe, plan, U, ib, bp
 
-    roofline["events"] = ("inside the timed region" if args.stage_events in ("gemm", "all") and not args.graph
+    roofline["events"] = ("inside the timed region" if stage_events in ("gemm", "all") and not o.graph
                           else "in the untimed steps after it")
     out = {
         "metric": "effective GFLOP/s over the conv stack (direct-conv FLOP count / time)",
-        "value": round(value, 1), "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": round(value, 1), "unit": "GFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": args.workload, "description": desc, "batch": N, "algorithm": algo,
-                   "per_layer": ",".join("im2col" if l.algo == "im2col" else "wino-" + l.pipe
-                                         for l in layers),
+        "config": {"workload": name, "description": desc, "batch": N, "algorithm": algo,
+                   "per_layer": ",".join("im2col" if l.algo == "im2col" else "wino-" + l.pipe for l in layers),
                    "filter_transform": "offline" if filter_ready else "online (inside the timed region)",
-                   "tuned": not args.no_tune, "stage_events": "none" if args.graph else args.stage_events,
-                   "launch": "hip graph replay" if args.graph else "per-layer calls",
+                   "tuned": bool(tune), "stage_events": "none" if o.graph else stage_events,
+                   "launch": "hip graph replay" if o.graph else "per-layer calls",
+                   "inputs": "uniform [-1,1), He-normal weights, the library's seeded xoshiro256** stream",
                    "device": info["arch"], "compute_units": info["compute_units"], "clock_mhz": info["clock_mhz"]},
         "roofline": roofline,
         "shader_clock": shader_clock,
         "transform_rooflines": transforms,
         "layers": per_layer,
     }
+    L.close()
+    return out
+
+
+def compact(r):
+    """What the `secondary` list keeps of a workload's result."""
+    rf = r["roofline"]
+    return {"workload": r["config"]["workload"], "description": r["config"]["description"],
+            "ms_per_step": r["ms_per_step"], "value": r["value"], "unit": r["unit"], "steps": r["steps"],
+            "warmup": r["warmup"], "tuned": r["config"]["tuned"], "per_layer": r["config"]["per_layer"],
+            "roofline": {k: rf.get(k) for k in ("kernel", "bound", "achieved", "peak", "unit", "frac", "events")}}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="vgg16_b32", choices=sorted(WORKLOADS))
+    ap.add_argument("--tune", action="store_true",
+                    help="search tile shape, pipeline and algorithm per layer before timing (default: the library's "
+                         "untuned choices; the stress workloads always search)")
+    ap.add_argument("--no-tune", action="store_true", help="(default behaviour, kept for older command lines)")
+    ap.add_argument("--offline-filter", action="store_true",
+                    help="transform the filters once outside the timed region")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="leave out the compact secondary workloads a default run appends")
+    ap.add_argument("--stage-events", default="auto", choices=["auto", "all", "gemm", "none"],
+                    help="which kernels are bracketed by events inside the timed region.  An event pair costs "
+                         "5-8 us per launch: 'gemm' brackets the dominant kernel only (the other kernels are "
+                         "bracketed in a few extra untimed steps), 'none' brackets nothing in the timed region "
+                         "(everything comes from the untimed steps).  'auto' (default) is 'gemm' while the "
+                         "brackets cost under 2 %% of a step (VGG-16 at batch 32: 9 launches in 3.5 ms), else "
+                         "'none' (ResNet-50: 53 launches, 15 %% of the step; batch-1 stacks)")
+    ap.add_argument("--pipeline", default="auto", choices=["auto", "staged", "fused", "onepass"],
+                    help="Winograd pipeline per layer: four staged kernels, GEMM + output transform fused, the "
+                         "single kernel, or what the library prefers for the layer (auto)")
+    ap.add_argument("--graph", action="store_true",
+                    help="record one step as a HIP graph and time replays of it (per-launch events are off; "
+                         "the default times the per-layer calls the reference's driver makes)")
+    ap.add_argument("--timed-only", action="store_true",
+                    help="no per-layer detail pass after the timed region and no secondary workloads (every launch "
+                         "of the process is then a warm-up or timed step: what a kernel trace of this command "
+                         "averages over)")
+    ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
+                    help="only run the plain copy kernel over MIB mebibytes (scale for the HBM traffic counters)")
+    args = ap.parse_args()
+    if args.copy_probe:
+        return copy_probe(args.copy_probe)
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (the layers shard by batch with no exchange step: "
+              "each GPU would hold the transformed filter and its share of the images); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    out = run_workload(args.workload, args.steps, args.warmup, args)
+    if args.workload == "vgg16_b32" and not (args.no_secondary or args.timed_only):
+        out["secondary"] = [compact(run_workload(w, min(args.steps, 20), args.warmup, args, detail=False))
+                            for w in SECONDARY]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
-    if shader_clock:
-        shader_clock["nominal_mhz"] = info["clock_mhz"]
-    L.close()
     print(json.dumps(out), flush=True)
 
 

@@ -81,6 +81,8 @@ _ABI = {
     "fc_graph_destroy": (C.c_int, [_vp]),
     "fc_maxpool2x2": (C.c_int, [_vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int]),
     "fc_device_copy": (C.c_int, [_vp, _vp, _vp, C.c_size_t]),
+    "fc_host_fill_uniform": (C.c_int, [C.c_uint64, C.c_float, C.c_float, _vp, C.c_size_t]),
+    "fc_host_fill_normal": (C.c_int, [C.c_uint64, C.c_float, _vp, C.c_size_t]),
     "fc_timing_enable": (C.c_int, [_vp, C.c_int]),
     "fc_timing_reset": (C.c_int, [_vp]),
     "fc_stage_time_ms": (C.c_int, [_vp, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_long)]),
@@ -140,6 +142,24 @@ def load_cdll():
         fn.restype = res
         fn.argtypes = args
     return lib
+
+
+def host_uniform(seed, shape, lo=-1.0, hi=1.0):
+    """Host array of the drivers' seeded uniform stream (no GPU needed)."""
+    out = np.empty(shape, np.float32)
+    rc = load_cdll().fc_host_fill_uniform(seed, lo, hi, out.ctypes.data_as(_vp), out.size)
+    if rc:
+        raise FastConvError(rc, "fc_host_fill_uniform")
+    return out
+
+
+def host_normal(seed, shape, sigma):
+    """Host array of the drivers' seeded normal stream (no GPU needed)."""
+    out = np.empty(shape, np.float32)
+    rc = load_cdll().fc_host_fill_normal(seed, sigma, out.ctypes.data_as(_vp), out.size)
+    if rc:
+        raise FastConvError(rc, "fc_host_fill_normal")
+    return out
 
 
 class Library:

@@ -5,6 +5,19 @@
 #include <new>
 
 #include "fc_internal.h"
+#include "../host/utility/rng.h"
+
+extern "C" int fc_host_fill_uniform(uint64_t seed, float lo, float hi, float *dst_host, size_t n) {
+    if (!dst_host && n) return FC_ERR_INVALID;
+    fastconv::FillUniform(seed, lo, hi, dst_host, n);
+    return FC_OK;
+}
+
+extern "C" int fc_host_fill_normal(uint64_t seed, float sigma, float *dst_host, size_t n) {
+    if (!dst_host && n) return FC_ERR_INVALID;
+    fastconv::FillNormal(seed, sigma, dst_host, n);
+    return FC_OK;
+}
 
 int fc_set_error(fc_context *ctx, int status, const char *what, hipError_t err) {
     if (ctx) {

@@ -104,6 +104,13 @@ int fc_fill_zero(fc_context *ctx, void *dst_dev, size_t bytes);
  * size must be multiples of 16. */
 int fc_device_copy(fc_context *ctx, void *dst_dev, const void *src_dev, size_t bytes);
 
+/* Synthetic inputs of the drivers, written to HOST memory: n floats uniform in [lo, hi), or
+ * normal with standard deviation sigma (Box-Muller in double), from a splitmix64-seeded
+ * xoshiro256** stream, so that every machine sees the same layer for a given seed.  Stand in
+ * for fillTestInput / fillTestKernel (ConvTest.cpp:18-46), which draw from rand(). */
+int fc_host_fill_uniform(uint64_t seed, float lo, float hi, float *dst_host, size_t n);
+int fc_host_fill_normal(uint64_t seed, float sigma, float *dst_host, size_t n);
+
 /* ---- stage timing (utility/helper.h:66-80 Timer, per stage) ----------- */
 
 /* stage_mask has bit (1 << stage) set for every stage whose kernel launches are

@@ -85,6 +85,13 @@ def test_winograd_width_limit_is_part_of_the_plan_and_of_the_auto_rule():
     assert lib.fc_prefer_winograd(C.byref(strided)) == 0
 
 
+def test_library_generator_is_the_oracle_generator():
+    import numpy as np
+    from oracle import oracle as O
+    assert np.array_equal(capi.host_uniform(7, (3, 333)), O.rng_uniform(7, (3, 333)))
+    assert np.array_equal(capi.host_normal(9, (1001,), 0.25), O.rng_normal(9, (1001,), 0.25))
+
+
 def test_no_gpu_means_a_loud_error_not_a_fallback():
     import pytest
     lib = capi.load_cdll()
