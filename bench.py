@@ -74,6 +74,9 @@ WORKLOADS = {
     "conv64_224_b32": (_w([(64, 64, 224, 1)]), 32, "winograd", "single 3x3 conv 64->64 @224, batch 32 (VGG-16 layer 2)"),
     "conv256_56_b32": (_w([(256, 256, 56, 1)]), 32, "winograd", "single 3x3 conv 256->256 @56, batch 32 (VGG-16 layers 6-7)"),
     "conv512_28_b32": (_w([(512, 512, 28, 1)]), 32, "winograd", "single 3x3 conv 512->512 @28, batch 32 (VGG-16 layers 9-10)"),
+    "igemm_3x3s2_b32": ([(128, 128, 56, 3, 2, 1, 1)], 32, "im2col", "single 3x3 stride-2 conv 128->128 @56, implicit GEMM, batch 32 (ResNet-50 conv3 entry)"),
+    "igemm_1x1_b32": ([(256, 64, 56, 1, 1, 0, 1)], 32, "im2col", "single 1x1 conv 256->64 @56, implicit GEMM, batch 32 (ResNet-50 bottleneck reduce)"),
+    "igemm_stem_b32": ([(3, 64, 224, 7, 2, 3, 1)], 32, "im2col", "single 7x7 stride-2 conv 3->64 @224, implicit GEMM, batch 32 (ResNet-50 stem)"),
     "stress_b64": (_w(STRESS), 64, "winograd", "VGG-16 256@56, 512@28, 512@14 at batch 64: staged (ZC) against blocked Winograd, tile shapes searched"),
     "stress_b128": (_w(STRESS), 128, "winograd", "VGG-16 256@56, 512@28, 512@14 at batch 128: staged (ZC) against blocked Winograd, tile shapes searched"),
 }

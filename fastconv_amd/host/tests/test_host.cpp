@@ -102,15 +102,35 @@ static void test_tuning_log() {
 
 static void test_select_algorithm() {
     nnp_size k3 = {3, 3}, k1 = {1, 1}, k7 = {7, 7}, s1 = {1, 1}, s2 = {2, 2};
-    nnp_size o56 = {56, 56}, o7 = {7, 7}, o224 = {224, 224};
+    nnp_size o56 = {56, 56}, o224 = {224, 224};
+    // the reference's skeleton (ConvTest.cpp:318-331)
     CHECK(select_algorithm(k1, s1, o56, 64, 256, 1) == nnp_convolution_algorithm_direct);
-    CHECK(select_algorithm(k3, s1, o56, 256, 256, 32) == nnp_convolution_algorithm_winograd);
     CHECK(select_algorithm(k3, s2, o56, 256, 256, 32) == nnp_convolution_algorithm_im2col);
     CHECK(select_algorithm(k1, s2, o56, 256, 512, 1) == nnp_convolution_algorithm_im2col);
     CHECK(select_algorithm(k7, s2, o224, 3, 64, 1) == nnp_convolution_algorithm_im2col);
-    CHECK(select_algorithm(k3, s1, o224, 3, 64, 32) == nnp_convolution_algorithm_im2col);     // 3 input channels
-    CHECK(select_algorithm(k3, s1, o7, 512, 512, 1) == nnp_convolution_algorithm_im2col);     // 4 tiles, 64x larger filter
-    CHECK(select_algorithm(k3, s1, o7, 512, 512, 32) == nnp_convolution_algorithm_winograd);
+    // 3x3 stride 1: the rule must pick the measured winner on every VGG-16 / ResNet-50 layer at batch 1
+    // and 32 (whole-layer milliseconds on MI355X, Winograd and implicit GEMM at their best tile shape);
+    // layers where the two are within 10 % of each other may go either way
+    static const struct { int c, k, h, n; double wino_ms, im2col_ms; } measured[] = {
+        {3, 64, 224, 1, 0.0249, 0.0113},     {64, 64, 224, 1, 0.0376, 0.0602},    {64, 128, 112, 1, 0.0319, 0.0411},
+        {128, 128, 112, 1, 0.0355, 0.0629},  {128, 256, 56, 1, 0.0323, 0.0411},   {256, 256, 56, 1, 0.0358, 0.0598},
+        {256, 512, 28, 1, 0.0322, 0.0404},   {512, 512, 28, 1, 0.0404, 0.0593},   {512, 512, 14, 1, 0.0405, 0.0354},
+        {64, 64, 56, 1, 0.0212, 0.0177},     {128, 128, 28, 1, 0.0204, 0.0196},   {256, 256, 14, 1, 0.0286, 0.0222},
+        {512, 512, 7, 1, 0.0405, 0.0230},    {3, 64, 224, 32, 0.2056, 0.1075},    {64, 64, 224, 32, 0.5019, 1.1918},
+        {64, 128, 112, 32, 0.2695, 0.5405},  {128, 128, 112, 32, 0.4366, 1.0763}, {128, 256, 56, 32, 0.2186, 0.5780},
+        {256, 256, 56, 32, 0.3398, 1.1469},  {256, 512, 28, 32, 0.1833, 0.6022},  {512, 512, 28, 32, 0.3069, 1.1825},
+        {512, 512, 14, 32, 0.1340, 0.3251},  {64, 64, 56, 32, 0.0570, 0.0952},    {128, 128, 28, 32, 0.0480, 0.1034},
+        {256, 256, 14, 32, 0.0540, 0.1002},  {512, 512, 7, 32, 0.0763, 0.1030}};
+    for (size_t i = 0; i < sizeof measured / sizeof measured[0]; i++) {
+        const nnp_size o = {(size_t)measured[i].h, (size_t)measured[i].h};
+        const bool wino = select_algorithm(k3, s1, o, measured[i].c, measured[i].k, measured[i].n) == nnp_convolution_algorithm_winograd;
+        const double ratio = measured[i].wino_ms / measured[i].im2col_ms;
+        if (ratio < 1.0 / 1.1) CHECK(wino);
+        if (ratio > 1.1) CHECK(!wino);
+    }
+    // wider than the Winograd input transform admits: implicit GEMM
+    nnp_size wide = {1021, 9};      // {width, height}
+    CHECK(select_algorithm(k3, s1, wide, 64, 64, 8) == nnp_convolution_algorithm_im2col);
 }
 
 static void test_conv_layer_geometry_and_naive() {

@@ -76,13 +76,16 @@ def test_plans_are_pure_host_arithmetic():
 def test_winograd_width_limit_is_part_of_the_plan_and_of_the_auto_rule():
     lib = capi.load_cdll()
     p = capi.WinoPlan()
-    ok = capi.ConvShape(1, 64, 9, 1020, 64, 3, 3, 1, 1, 1, 1, 1, 1)
-    wide = capi.ConvShape(1, 64, 9, 1021, 64, 3, 3, 1, 1, 1, 1, 1, 1)
+    ok = capi.ConvShape(8, 64, 9, 1020, 64, 3, 3, 1, 1, 1, 1, 1, 1)
+    wide = capi.ConvShape(8, 64, 9, 1021, 64, 3, 3, 1, 1, 1, 1, 1, 1)
     assert lib.fc_wino_make_plan(C.byref(ok), 0, C.byref(p)) == 0 and p.tiles_w == 170
     assert lib.fc_wino_make_plan(C.byref(wide), 0, C.byref(p)) == -6
     assert lib.fc_prefer_winograd(C.byref(ok)) == 1 and lib.fc_prefer_winograd(C.byref(wide)) == 0
-    strided = capi.ConvShape(1, 64, 56, 56, 64, 3, 3, 2, 2, 1, 1, 1, 1)
+    strided = capi.ConvShape(8, 64, 56, 56, 64, 3, 3, 2, 2, 1, 1, 1, 1)
     assert lib.fc_prefer_winograd(C.byref(strided)) == 0
+    few_channels = capi.ConvShape(32, 3, 224, 224, 64, 3, 3, 1, 1, 1, 1, 1, 1)
+    little_work = capi.ConvShape(1, 512, 14, 14, 512, 3, 3, 1, 1, 1, 1, 1, 1)
+    assert lib.fc_prefer_winograd(C.byref(few_channels)) == 0 and lib.fc_prefer_winograd(C.byref(little_work)) == 0
 
 
 def test_library_generator_is_the_oracle_generator():
