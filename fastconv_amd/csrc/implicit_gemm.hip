@@ -140,8 +140,15 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm0 = (wave / TL::WGN_) * TL::WM, wn0 = (wave % TL::WGN_) * TL::WN;
-    // output-channel blocks innermost: neighbouring workgroups share the gathered pixels
-    const int pb = blockIdx.x / p.nKB, kb = blockIdx.x - pb * p.nKB;
+    // Workgroups are dealt to the 8 XCDs round-robin by linear id, and every XCD has an L2 of its own.
+    // Tiles are numbered pixel block major, output-channel block minor, and every XCD owns a contiguous
+    // eighth of that sequence: the output-channel blocks that share one block of gathered pixels run
+    // side by side on ONE XCD and find the pixels in its L2 (dealt round-robin, every XCD would fetch
+    // every pixel block: measured 4-6x the algorithmic traffic on the ResNet-50 projections).
+    const int nTiles = p.nKB * p.nPB, perXcd = (nTiles + 7) >> 3;
+    const int tileId = (blockIdx.x & 7) * perXcd + (blockIdx.x >> 3);
+    if ((int)(blockIdx.x >> 3) >= perXcd || tileId >= nTiles) return;
+    const int pb = tileId / p.nKB, kb = tileId - pb * p.nKB;
 
     // filter tile: straight 16-byte copies
     const int arow = tid / (BM / 4), acol = (tid % (BM / 4)) * 4;
@@ -392,7 +399,7 @@ const int kNumIgConfigs = sizeof(kIgConfigs) / sizeof(kIgConfigs[0]);
 
 template <class TL>
 void launch(fc_context *ctx, IgemmParams &p) {
-    const dim3 grid((unsigned)(p.nKB * p.nPB), (unsigned)p.splitK);
+    const dim3 grid((unsigned)(((p.nKB * p.nPB + 7) / 8) * 8), (unsigned)p.splitK);
     const bool pointwise = p.kh == 1 && p.kw == 1 && p.sh == 1 && p.sw == 1 && p.pt == 0 && p.pl == 0 &&
                            p.OH == p.H && p.OW == p.W && (p.H * p.W) % 4 == 0 && p.C % TL::BK_ == 0 &&
                            ((uintptr_t)p.x & 15) == 0;
