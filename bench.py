@@ -204,6 +204,7 @@ def tune_layer(L, lay, V, M, scratch_bytes, iters=3, full_search=False):
 
     def note(cls, cfg, pipe, ms, ib):
         nonlocal best
+        log("  candidate %s: %s cfg %s images/block %d: %.4f ms" % (lay.name(), pipe, cfg, ib, ms))
         if ms < best[2]:
             best = (cfg, pipe, ms, ib)
         if cls not in per_class or ms < per_class[cls]["ms"]:

@@ -53,6 +53,7 @@ struct IgemmParams {
     int nKB, nPB;
     int splitK, stagesPerSplit;   // reduction split over blockIdx.y; partial sums go to ws
     float *ws;                    // [splitK][K][Npix] when splitK > 1
+    long xBytes;                  // size of the input tensor
     int fastStore;                // K is a whole number of tiles, every output byte offset fits 32 bits, bias 16-byte aligned
     fc_fastdiv divOHW, divOW;
 };
@@ -97,8 +98,7 @@ __device__ __forceinline__ void ig_store_rows(float *lds, const floatx4 (&r)[siz
 // instead) and its value is not touched here: whether it counts is recorded as bit `slot`
 // of `okBits` and applied when the element is written to LDS, so that the loads of a
 // stage stay in flight under the MFMAs of the stage before.
-// MASKED = false: every tap of every output pixel lies inside the image (no padding on the top
-// and left, and the last window ends inside) and the reduction has no padding rows: no test.
+// MASKED = false: no test at all (kept for completeness; the buffer modes below serve such layers).
 template <bool MASKED>
 __device__ __forceinline__ float ig_gather(const float *ximg, int pixOff, uint32_t maskR, uint32_t maskS,
                                            const int32_t *table, int kred, int slot, uint32_t &okBits) {
@@ -123,8 +123,35 @@ __device__ __forceinline__ void ig_scatter_rows(float *lds, const float (&r)[siz
     ((lds[I * rowStride] = (!MASKED || ((okBits >> I) & 1u)) ? r[I] : 0.f), ...);
 }
 
-// How the B tile (a slice of the column matrix) reaches LDS.
-enum { IG_GATHER = 0, IG_POINTWISE = 1, IG_GATHER_INSIDE = 2 };
+// The same element through a buffer resource over the whole input tensor (tensors below 2 GiB): the
+// address is one 32-bit byte offset from a scalar base, and a tap outside the image gets bit 31 of
+// its offset set, which puts it past the end of the buffer: the hardware's range check returns 0
+// for it without touching memory.  No 64-bit address arithmetic, no select at the LDS write.
+// invLo / invHi: bit t = r*kw + s is set when tap (r, s) of this thread's pixel lies outside the
+// image (taps 64 and up, which only padding rows of the reduction name, count as outside).
+template <bool MASKED>
+__device__ __forceinline__ float ig_gather_buf(__amdgpu_buffer_rsrc_t xres, uint32_t pixByte, uint32_t invLo, uint32_t invHi,
+                                               const int32_t *table, int kred, int kw) {
+    uint32_t voff = pixByte + 4u * (uint32_t)table[2 * kred];
+    if (MASKED) {
+        const int rs = table[2 * kred + 1];
+        const uint32_t t = (uint32_t)(rs >> 16) * (uint32_t)kw + (uint32_t)(rs & 0xffff);     // wave-uniform
+        const uint32_t word = t < 32u ? invLo : invHi;
+        const uint32_t bad = t < 64u ? (word >> (t & 31u)) & 1u : 1u;
+        voff |= bad << 31;
+    }
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xres, voff, 0, 0));
+}
+template <bool MASKED, int... I>
+__device__ __forceinline__ void ig_gather_rows_buf(float (&r)[sizeof...(I)], __amdgpu_buffer_rsrc_t xres, uint32_t pixByte,
+                                                   uint32_t invLo, uint32_t invHi, const int32_t *table, int kred0, int rowStep,
+                                                   int kw, std::integer_sequence<int, I...>) {
+    ((r[I] = ig_gather_buf<MASKED>(xres, pixByte, invLo, invHi, table, kred0 + I * rowStep, kw)), ...);
+}
+
+// How the B tile (a slice of the column matrix) reaches LDS.  IG_GATHER is the fallback of the two
+// buffer modes for input tensors of 2 GiB and more.
+enum { IG_GATHER = 0, IG_POINTWISE = 1, IG_BUF_MASKED = 2, IG_BUF_INSIDE = 3 };
 
 // PW: pointwise layers (1x1, stride 1, no padding: the column matrix IS the input, row c of it
 // is channel c of x, contiguous over the pixels) whose pixels-per-image count is a multiple of 4
@@ -132,7 +159,7 @@ enum { IG_GATHER = 0, IG_POINTWISE = 1, IG_GATHER_INSIDE = 2 };
 // a pixel group past the end re-reads the last group (its columns are never stored).
 template <class TL, int MODE>
 __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(const IgemmParams p) {
-    constexpr bool PW = MODE == IG_POINTWISE, MASKED = MODE != IG_GATHER_INSIDE;
+    constexpr bool PW = MODE == IG_POINTWISE, BUF = MODE == IG_BUF_MASKED || MODE == IG_BUF_INSIDE;
     constexpr int BM = TL::BM_, BN = TL::BN_, BK = TL::BK_;
     constexpr int MI = TL::MI, NI = TL::NI, A_LD = TL::A_LD, B_LD = TL::B_LD;
     __shared__ __attribute__((aligned(16))) float As[2][BK * BM];
@@ -174,6 +201,23 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
         for (int r = 0; r < p.kh; r++) maskR |= ((unsigned)(ih0 + r) < (unsigned)p.H) ? (1u << r) : 0u;
         for (int q = 0; q < p.kw; q++) maskS |= ((unsigned)(iw0 + q) < (unsigned)p.W) ? (1u << q) : 0u;
     }
+    // buffer modes: byte offset of the window origin in the whole tensor, and the taps outside the image
+    uint32_t pixByte = 0, invLo = ~0u, invHi = ~0u;
+    __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.x), 0, BUF ? (int)p.xBytes : 0, 0x00020000);
+    if (BUF && pix < p.Npix) {
+        pixByte = 4u * (uint32_t)((long)(ximg - p.x) + pixOff);
+        if (MODE == IG_BUF_MASKED) {
+            const uint32_t rowBits = ~maskS & ((1u << p.kw) - 1u);      // taps of one window row outside the image
+            uint64_t inv = 0;
+            for (int r = 0; r < p.kh; r++) {
+                const uint32_t bits = ((maskR >> r) & 1u) ? rowBits : ((1u << p.kw) - 1u);
+                if (r * p.kw < 64) inv |= (uint64_t)bits << (r * p.kw);
+            }
+            if (p.kh * p.kw < 64) inv |= ~0ull << (p.kh * p.kw);
+            invLo = (uint32_t)inv;
+            invHi = (uint32_t)(inv >> 32);
+        }
+    }
     const int bLds = grow0 * BN + gcol;
 
     // pointwise: this thread's 4-pixel column group and first row of each copy pass
@@ -205,8 +249,10 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
     if (PW) {
         vg += (size_t)sBegin * vStage;
         ig_load_rows(rv, vg, vPass, SeqBV());
+    } else if (BUF) {
+        ig_gather_rows_buf<MODE == IG_BUF_MASKED>(rb, xres, pixByte, invLo, invHi, p.table, sBegin * BK + grow0, TL::ROW_STEP, p.kw, SeqB());
     } else {
-        rbOk = ig_gather_rows<MASKED>(rb, ximg, pixOff, maskR, maskS, p.table, sBegin * BK + grow0, TL::ROW_STEP, SeqB());
+        rbOk = ig_gather_rows<true>(rb, ximg, pixOff, maskR, maskS, p.table, sBegin * BK + grow0, TL::ROW_STEP, SeqB());
     }
 
     floatx16 acc[MI][NI];
@@ -219,12 +265,13 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
 
     ig_store_rows(&As[0][aLds], ra, TL::A_ROWS * BM, SeqA());
     if (PW) ig_store_rows(&Bs[0][vLds], rv, BV_ROWS * BN, SeqBV());
-    else ig_scatter_rows<MASKED>(&Bs[0][bLds], rb, rbOk, TL::ROW_STEP * BN, SeqB());
+    else ig_scatter_rows<!BUF>(&Bs[0][bLds], rb, rbOk, TL::ROW_STEP * BN, SeqB());
     // stage s of the reduction into the staging registers
     auto load_stage = [&](const int s) __attribute__((always_inline)) {
         ig_load_rows(ra, ag + (size_t)(s - sBegin) * aStage, aPass, SeqA());
         if (PW) ig_load_rows(rv, vg + (size_t)(s - sBegin) * vStage, vPass, SeqBV());
-        else rbOk = ig_gather_rows<MASKED>(rb, ximg, pixOff, maskR, maskS, p.table, s * BK + grow0, TL::ROW_STEP, SeqB());
+        else if (BUF) ig_gather_rows_buf<MODE == IG_BUF_MASKED>(rb, xres, pixByte, invLo, invHi, p.table, s * BK + grow0, TL::ROW_STEP, p.kw, SeqB());
+        else rbOk = ig_gather_rows<true>(rb, ximg, pixOff, maskR, maskS, p.table, s * BK + grow0, TL::ROW_STEP, SeqB());
     };
     if (sBegin + 1 < sEnd) load_stage(sBegin + 1);
     __syncthreads();
@@ -266,7 +313,7 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
                 // and the one after it is requested at once: a whole stage in flight
                 ig_store_rows(&As[buf ^ 1][aLds], ra, TL::A_ROWS * BM, SeqA());
                 if (PW) ig_store_rows(&Bs[buf ^ 1][vLds], rv, BV_ROWS * BN, SeqBV());
-                else ig_scatter_rows<MASKED>(&Bs[buf ^ 1][bLds], rb, rbOk, TL::ROW_STEP * BN, SeqB());
+                else ig_scatter_rows<!BUF>(&Bs[buf ^ 1][bLds], rb, rbOk, TL::ROW_STEP * BN, SeqB());
                 if (s + 2 < sEnd) load_stage(s + 2);
             }
         }
@@ -406,8 +453,11 @@ void launch(fc_context *ctx, IgemmParams &p) {
     // no tap of any window leaves the image, and no padding rows in the reduction
     const bool inside = p.pt == 0 && p.pl == 0 && (p.OH - 1) * p.sh + p.kh <= p.H && (p.OW - 1) * p.sw + p.kw <= p.W &&
                         (p.C * p.kh * p.kw) % TL::BK_ == 0;
+    // one 32-bit byte offset with bit 31 to spare reaches every element of the tensor
+    const bool buffer = p.xBytes < (1l << 31);
     if (pointwise) igemm_conv_kernel<TL, IG_POINTWISE><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
-    else if (inside) igemm_conv_kernel<TL, IG_GATHER_INSIDE><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
+    else if (buffer && inside) igemm_conv_kernel<TL, IG_BUF_INSIDE><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
+    else if (buffer && p.kh * p.kw <= 64) igemm_conv_kernel<TL, IG_BUF_MASKED><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);      // the taps of a window are one 64-bit mask
     else igemm_conv_kernel<TL, IG_GATHER><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
 }
 
@@ -588,6 +638,7 @@ static int igemm_run(fc_context *ctx, const fc_igemm_plan *plan, const float *x_
     p.N = s.N; p.C = s.C; p.H = s.H; p.W = s.W; p.K = s.K; p.OH = plan->OH; p.OW = plan->OW;
     p.kh = s.kh; p.kw = s.kw; p.sh = s.sh; p.sw = s.sw; p.pt = s.pt; p.pl = s.pl; p.relu = relu;
     p.Kred_pad = plan->Kred_pad; p.K_pad = plan->K_pad; p.Npix = plan->Npix;
+    p.xBytes = 4l * s.N * s.C * s.H * s.W;
     p.nKB = plan->K_pad / cfg.bm;
     p.nPB = (int)((plan->Npix + cfg.bn - 1) / cfg.bn);
     p.divOHW = fc_make_fastdiv((uint32_t)(plan->OH * plan->OW));

@@ -323,6 +323,8 @@ IGEMM_SHAPES = [
     (32, 256, 56, 56, 64, 1, 1, 1, 1, 0), (32, 512, 28, 28, 128, 1, 1, 1, 1, 0), (32, 2048, 7, 7, 512, 1, 1, 1, 1, 0),
     (32, 1024, 14, 14, 256, 1, 1, 1, 1, 0), (32, 128, 56, 56, 128, 3, 3, 2, 2, 1), (32, 256, 28, 28, 256, 3, 3, 2, 2, 1),
     (32, 512, 14, 14, 512, 3, 3, 2, 2, 1), (8, 3, 224, 224, 64, 7, 7, 2, 2, 3),
+    # windows of 63, 64 (one 64-bit tap mask) and 81 taps (beyond it: the pointer gather)
+    (2, 3, 20, 21, 8, 7, 9, 1, 1, 3), (1, 4, 19, 19, 9, 8, 8, 2, 2, 4), (2, 3, 20, 20, 8, 9, 9, 1, 1, 4),
 ]
 
 
@@ -334,6 +336,28 @@ def test_implicit_gemm_against_oracle(lib, shp):
     y = lib.implicit_gemm_conv(cshape(s), x, w)
     assert O.max_rel_err(y, O.naive_conv_f64(s, x, w)) <= TOL_IM2COL
     assert O.max_rel_err(y, O.naive_conv_f32(s, x, w)) <= TOL_IM2COL
+
+
+def test_implicit_gemm_input_of_2_gib_takes_the_pointer_gather(lib):
+    """Inputs below 2 GiB are gathered through a buffer resource with 32-bit offsets; a larger one
+    falls back to 64-bit pointers.  One tap per filter gives an exact answer at this size."""
+    import fastconv_amd as F
+    N, C, H, W, K = 1, 8, 8200, 8200, 2
+    assert 4 * N * C * H * W >= 1 << 31
+    s = O.shape(N, C, H, W, K)
+    x = O.rng_uniform(5, (N, C, H, W))
+    w = np.zeros((K, C, 3, 3), np.float32)
+    w[0, 3, 0, 2] = 1.0
+    w[1, 7, 2, 1] = 1.0
+    big = F.load(0, 5 << 30)
+    try:
+        y = big.implicit_gemm_conv(cshape(s), x, w)
+    finally:
+        big.close()
+    xp = np.pad(x[0, 3], 1)
+    assert np.array_equal(y[0, 0], xp[0:H, 2:2 + W])
+    xp = np.pad(x[0, 7], 1)
+    assert np.array_equal(y[0, 1], xp[2:2 + H, 1:1 + W])
 
 
 def test_implicit_gemm_asymmetric_padding_and_bias(lib):
