@@ -23,6 +23,17 @@ def test_host_unit_tests_pass():
     assert "all host tests passed" in r.stdout
 
 
+def test_host_unit_tests_pass_under_address_and_undefined_behaviour_sanitizers():
+    """The pools, the range allocator, the tuning log and the naive layer are pointer-heavy host code:
+    the same unit tests, built with -fsanitize=address,undefined (host code only)."""
+    subprocess.check_call(["make", "-C", PKG, "-s", "hosttest-san"])
+    env = dict(os.environ, ASAN_OPTIONS="verify_asan_link_order=0:abort_on_error=1", UBSAN_OPTIONS="halt_on_error=1")
+    r = subprocess.run([os.path.join(PKG, "bin", "test_host_san")], capture_output=True, text=True, timeout=300, env=env)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "all host tests passed" in r.stdout
+    assert "ERROR: AddressSanitizer" not in r.stderr and "runtime error" not in r.stderr
+
+
 def test_driver_generator_matches_oracle_generator_bit_for_bit():
     exe = _build()
     r = subprocess.run([exe], capture_output=True, text=True, timeout=120,
