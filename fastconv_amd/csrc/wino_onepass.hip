@@ -37,7 +37,8 @@ constexpr int kKB = 64;                         // output channels per workgroup
 constexpr int kTmpTile = 68;                    // floats per (channel, tile) block of tmp: 16-byte aligned rows,
                                                 // 17 quads so that lanes on consecutive tiles spread over the banks
 constexpr int kTmpFloats = kCB * kTB * kTmpTile;        // one buffer
-constexpr int kVsFreq = 80;                     // floats per frequency of Vs (64 used): see the store pattern below
+constexpr int kVsFreq = 72;                     // floats per frequency of Vs (64 used): 8 banks on, so that the four
+                                                // patch columns a half-wavefront stores land in four different bank octets
 constexpr int kVsFloats = 64 * kVsFreq;         // one buffer
 constexpr int kMlTile = 36;                     // floats per (frequency, tile) of the exchange buffer: 32 channels, padded
 constexpr size_t kOnePassLdsBytes = (size_t)64 * kTB * kMlTile * sizeof(float);      // 144 KiB
@@ -93,8 +94,10 @@ __global__ __launch_bounds__(kFusedThreads, 1) void wino_onepass_kernel(const On
     const size_t chunkX = (size_t)kCB * p.H * p.W;
     const int tmpW = (c1 * kTB + tl1) * kTmpTile + i1 * 8;
 
-    // ---- step 2: thread = column j2 of tile tl2, channel c2 (a wavefront: 16 tiles x 4 columns)
-    const int tl2 = tid & 15, j2 = (tid >> 4) & 7, c2 = tid >> 7;
+    // ---- step 2: thread = column j2 of tile tl2, channel c2 (a wavefront: 16 tiles x 4 columns).  Lanes
+    // 0..31 hold tiles 0..7 x 4 columns, lanes 32..63 tiles 8..15: with 17 quads per tile in tmp and
+    // kVsFreq floats per frequency in Vs, the 32 lanes LDS serves together hit 32 different banks in both.
+    const int tl2 = (lane & 7) | ((lane >> 5) << 3), j2 = ((lane >> 3) & 3) + 4 * (wave & 1), c2 = wave >> 1;
     const int tmpR = (c2 * kTB + tl2) * kTmpTile + j2;
     const int vsW = j2 * kVsFreq + c2 * kTB + tl2;            // + 8*kVsFreq per output row
 
@@ -103,7 +106,9 @@ __global__ __launch_bounds__(kFusedThreads, 1) void wino_onepass_kernel(const On
     const int nq = p.C_pad / kCB;                             // even
     const size_t chunkU = (size_t)p.nKB * 256;                // floats per (frequency, chunk)
     const size_t planeU = (size_t)nq * chunkU;                // floats per frequency
-    const float *ub = p.U + (size_t)(wv * kFW) * planeU + (size_t)kb * 256 + lane * 4;
+    // wave-uniform base (scalar registers) + one 32-bit lane offset: the filter loads need no address arithmetic
+    const float *ub = p.U + (size_t)(wv * kFW) * planeU + (size_t)kb * 256;
+    const uint32_t ubLane = (uint32_t)lane * 16u;
     const int vsR = wv * kFW * kVsFreq + lane;                // + kVsFreq per frequency
 
     floatx4 acc[kFW][4];
@@ -129,7 +134,8 @@ __global__ __launch_bounds__(kFusedThreads, 1) void wino_onepass_kernel(const On
     auto loadU = [&](int q, floatx4 (&dst)[kFW]) {
         const float *src = ub + (size_t)q * chunkU;
 #pragma unroll
-        for (int f = 0; f < kFW; f++) dst[f] = *reinterpret_cast<const floatx4 *>(src + f * planeU);
+        for (int f = 0; f < kFW; f++)
+            dst[f] = *reinterpret_cast<const floatx4 *>(reinterpret_cast<const char *>(src + f * planeU) + ubLane);
     };
     // window (chunk q) -> patch row -> B along the row -> tmp[buf].  Rows that touch the image
     // border are shifted and zero-filled through a private 8-float slot of LDS.
@@ -225,7 +231,9 @@ __global__ __launch_bounds__(kFusedThreads, 1) void wino_onepass_kernel(const On
                 *reinterpret_cast<floatx4 *>(Ml + ((wave * kFW + f) * 16 + (lane & 15)) * kMlTile + s2 * 16 + 4 * (lane >> 4)) =
                     acc[f][half * 2 + s2];
         __syncthreads();
-        const int krow = tid >> 4, tl = tid & 15;
+        // 32 channels x 16 tiles per half; lanes 0..31 of a wavefront hold tiles 0..7 x 4 channels (bank-conflict
+        // free reads of the exchange buffer, whose tiles are 36 floats apart)
+        const int krow = 4 * wave + ((lane >> 3) & 3), tl = (lane & 7) | ((lane >> 5) << 3);
         const int k = kb * kKB + half * 32 + krow;
         const uint32_t t = (uint32_t)tb * kTB + tl;
         if (k < p.out.K && t < (uint32_t)p.out.T) {
