@@ -134,3 +134,30 @@ def test_struct_layouts_match_the_header(tmp_path):
         seen += 1
     assert seen == sum(len(ct._fields_) + 1 for ct in structs.values())
     assert len(capi.STAGE_NAMES) == 8       # FC_STAGE_COUNT
+
+
+def test_bench_reads_measured_traffic_from_the_committed_profile():
+    """bench.py takes roofline.traffic from profiles/gemm_hbm_traffic_pmc.txt: every GEMM launch of the
+    default workload (library choices) must be in it, with a plausible ratio to the algorithmic bytes."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    table = bench.measured_traffic()
+    assert table, "profiles/gemm_hbm_traffic_pmc.txt has no traffic lines"
+    lib = capi.load_cdll()
+    layers, N, algo, _ = bench.WORKLOADS["vgg16_b32"]
+    seen = 0
+    for (Cc, K, H, ks, st, pad, rep) in layers:
+        s = capi.ConvShape(N, Cc, H, H, K, ks, ks, st, st, pad, pad, pad, pad)
+        if lib.fc_wino_prefer_onepass(C.byref(s)) or lib.fc_wino_prefer_fused(C.byref(s)):
+            continue                                   # no staged GEMM launch for this layer
+        g = capi.GemmConfig()
+        assert lib.fc_wino_gemm_get_config(lib.fc_wino_gemm_default_config(C.byref(s)), C.byref(g)) == 0
+        key = ("wino_gemm_kernel", N, Cc, K, H, 3, 1, "%dx%dx%d" % (g.bm, g.bn, g.bk))
+        assert key in table, key
+        T = N * ((H + 5) // 6) ** 2
+        algorithmic = 256.0 * (K * Cc + Cc * T + K * T)
+        assert 0.95 <= table[key] / algorithmic <= 1.25, (key, table[key] / algorithmic)
+        seen += 1
+    assert seen >= 5
