@@ -80,7 +80,8 @@ WORKLOADS = {
     "stress_b64": (_w(STRESS), 64, "winograd", "VGG-16 256@56, 512@28, 512@14 at batch 64: staged (ZC) against blocked Winograd, tile shapes searched"),
     "stress_b128": (_w(STRESS), 128, "winograd", "VGG-16 256@56, 512@28, 512@14 at batch 128: staged (ZC) against blocked Winograd, tile shapes searched"),
 }
-SECONDARY = ("vgg16_b1", "resnet50_b32", "im2col_abc_b1")
+# (workload, filter transform offline): compact results a default run appends
+SECONDARY = (("vgg16_b1", False), ("vgg16_b1", True), ("resnet50_b32", False), ("im2col_abc_b1", False))
 
 ST_KT, ST_IT, ST_GEMM, ST_OT, ST_IGEMM, ST_FUSED, ST_ONEPASS = 0, 1, 2, 3, 4, 6, 7
 
@@ -278,7 +279,7 @@ def cpu_baseline(target_seconds=3.0):
         return total_flops, total_s
 
     fl, s1 = run(1)
-    batch = int(max(1, min(32, (target_seconds - s1) // max(s1, 1e-3))))
+    batch = int(max(1, min(32, target_seconds // max(s1, 1e-3))))
     if batch > 1:
         fl, s1 = run(batch)
     return {"value": round(fl / s1 / 1e9, 2), "unit": "GFLOP/s", "cores": cores, "kind": "port",
@@ -323,7 +324,7 @@ def measured_traffic():
     return out
 
 
-def run_workload(name, steps, warmup, o, detail=True):
+def run_workload(name, steps, warmup, o, detail=True, offline_filter=None):
     """Builds the layers of one workload on the device, times `steps` steps and returns the result fields."""
     import fastconv_amd as F
     layers_def, N, algo, desc = WORKLOADS[name]
@@ -393,7 +394,7 @@ def run_workload(name, steps, warmup, o, detail=True):
                    " (winograd %.3f ms)" % wres[2] if wres else ""))
     L.sync()
 
-    filter_ready = o.offline_filter
+    filter_ready = o.offline_filter if offline_filter is None else offline_filter
 
     def step():
         for lay in layers:
@@ -730,6 +731,7 @@ def compact(r):
     return {"workload": r["config"]["workload"], "description": r["config"]["description"],
             "ms_per_step": r["ms_per_step"], "value": r["value"], "unit": r["unit"], "steps": r["steps"],
             "warmup": r["warmup"], "tuned": r["config"]["tuned"], "per_layer": r["config"]["per_layer"],
+            "filter_transform": r["config"]["filter_transform"],
             "roofline": {k: rf.get(k) for k in ("kernel", "bound", "achieved", "peak", "unit", "frac", "events")}}
 
 
@@ -777,8 +779,8 @@ def main():
 
     out = run_workload(args.workload, args.steps, args.warmup, args)
     if args.workload == "vgg16_b32" and not (args.no_secondary or args.timed_only):
-        out["secondary"] = [compact(run_workload(w, min(args.steps, 20), args.warmup, args, detail=False))
-                            for w in SECONDARY]
+        out["secondary"] = [compact(run_workload(w, min(args.steps, 20), args.warmup, args, detail=False,
+                                                 offline_filter=off)) for (w, off) in SECONDARY]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out), flush=True)
