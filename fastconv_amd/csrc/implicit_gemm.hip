@@ -17,27 +17,42 @@ namespace {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));   // native vector: arrays of it stay in registers
 
-// Row table entry for reduction index kred = (c*kh + r)*kw + s:
+// Order of the reduction index.  Channel-major (the column-matrix rows of
+// convLayer/im2colConv.cpp:285-309): kred = (c*kh + r)*kw + s.  Tap-major, used whenever the channel
+// count is a whole number of LDS stages (C % BK == 0): kred = (r*kw + s)*C + c, so that the BK rows of a
+// stage share one filter tap -- one in-image test and one window offset per stage instead of one per
+// gathered element, and consecutive rows are consecutive channels (no table lookups in the loop).
+// The packed filter and the row table follow whichever order the layer uses.
+// Row table entry for reduction row kred (tap (r, s) of channel c):
 //   [2*kred]   = c*H*W + r*W + s      (offset from the window origin)
 //   [2*kred+1] = r << 16 | s          (31 << 16 | 31 for padding rows: a mask bit that is never set)
 __global__ __launch_bounds__(256) void igemm_pack_filter_kernel(const float *__restrict__ w,
                                                                 float *__restrict__ Wp,
                                                                 int32_t *__restrict__ table, int K, int C,
                                                                 int kh, int kw, int H, int W, int Kred,
-                                                                int Kred_pad, int K_pad) {
+                                                                int Kred_pad, int K_pad, int tapMajor) {
     const int k = blockIdx.x * 64 + (threadIdx.x & 63);
     const int kred = blockIdx.y * 4 + (threadIdx.x >> 6);
     if (kred >= Kred_pad) return;
-    if (k < K_pad) Wp[(size_t)kred * K_pad + k] = (k < K && kred < Kred) ? w[(size_t)k * Kred + kred] : 0.f;
-    if (blockIdx.x == 0 && (threadIdx.x & 63) == 0) {
-        if (kred < Kred) {
-            const int c = kred / (kh * kw), rs = kred - c * kh * kw, r = rs / kw, s = rs - r * kw;
-            table[2 * kred] = c * H * W + r * W + s;
-            table[2 * kred + 1] = (r << 16) | s;
+    int c = 0, r = 31, s = 31;
+    if (kred < Kred) {
+        if (tapMajor) {
+            const int t = kred / C;
+            c = kred - t * C;
+            r = t / kw;
+            s = t - r * kw;
         } else {
-            table[2 * kred] = 0;
-            table[2 * kred + 1] = (31 << 16) | 31;
+            c = kred / (kh * kw);
+            const int rs = kred - c * kh * kw;
+            r = rs / kw;
+            s = rs - r * kw;
         }
+    }
+    if (k < K_pad)
+        Wp[(size_t)kred * K_pad + k] = (k < K && kred < Kred) ? w[((size_t)k * C + c) * (kh * kw) + r * kw + s] : 0.f;
+    if (blockIdx.x == 0 && (threadIdx.x & 63) == 0) {
+        table[2 * kred] = kred < Kred ? c * H * W + r * W + s : 0;
+        table[2 * kred + 1] = (r << 16) | s;
     }
 }
 
@@ -151,7 +166,8 @@ __device__ __forceinline__ void ig_gather_rows_buf(float (&r)[sizeof...(I)], __a
 
 // How the B tile (a slice of the column matrix) reaches LDS.  IG_GATHER is the fallback of the two
 // buffer modes for input tensors of 2 GiB and more.
-enum { IG_GATHER = 0, IG_POINTWISE = 1, IG_BUF_MASKED = 2, IG_BUF_INSIDE = 3 };
+// IG_TAP_*: the buffer gather for tap-major layers (see igemm_pack_filter_kernel).
+enum { IG_GATHER = 0, IG_POINTWISE = 1, IG_BUF_MASKED = 2, IG_TAP_MASKED = 3, IG_TAP_INSIDE = 4 };
 
 // PW: pointwise layers (1x1, stride 1, no padding: the column matrix IS the input, row c of it
 // is channel c of x, contiguous over the pixels) whose pixels-per-image count is a multiple of 4
@@ -159,7 +175,8 @@ enum { IG_GATHER = 0, IG_POINTWISE = 1, IG_BUF_MASKED = 2, IG_BUF_INSIDE = 3 };
 // a pixel group past the end re-reads the last group (its columns are never stored).
 template <class TL, int MODE>
 __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(const IgemmParams p) {
-    constexpr bool PW = MODE == IG_POINTWISE, BUF = MODE == IG_BUF_MASKED || MODE == IG_BUF_INSIDE;
+    constexpr bool PW = MODE == IG_POINTWISE, TAP = MODE == IG_TAP_MASKED || MODE == IG_TAP_INSIDE;
+    constexpr bool BUF = MODE == IG_BUF_MASKED || TAP;
     constexpr int BM = TL::BM_, BN = TL::BN_, BK = TL::BK_;
     constexpr int MI = TL::MI, NI = TL::NI, A_LD = TL::A_LD, B_LD = TL::B_LD;
     __shared__ __attribute__((aligned(16))) float As[2][BK * BM];
@@ -206,7 +223,7 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
     __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.x), 0, BUF ? (int)p.xBytes : 0, 0x00020000);
     if (BUF && pix < p.Npix) {
         pixByte = 4u * (uint32_t)((long)(ximg - p.x) + pixOff);
-        if (MODE == IG_BUF_MASKED) {
+        if (MODE == IG_BUF_MASKED || MODE == IG_TAP_MASKED) {
             const uint32_t rowBits = ~maskS & ((1u << p.kw) - 1u);      // taps of one window row outside the image
             uint64_t inv = 0;
             for (int r = 0; r < p.kh; r++) {
@@ -244,13 +261,48 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
     // this block's share of the reduction
     const int nStagesAll = p.Kred_pad / BK;
     const int sBegin = blockIdx.y * p.stagesPerSplit, sEnd = min(sBegin + p.stagesPerSplit, nStagesAll);
+    // Tap-major gather: the BK rows of a stage are channels tapC .. tapC+BK-1 of one tap (tapR, tapS).
+    // Stages are gathered in order, so the tap and the channel are running counters, wave-uniform
+    // (scalar registers); only the last addition of an element's offset is per lane.
+    const uint32_t chanStep = 4u * (uint32_t)(p.H * p.W);
+    int tapT = 0, tapR = 0, tapS = 0, tapC = 0;
+    if (TAP) {
+        const int stagesPerTap = p.C / BK;          // tap-major layers only: C % BK == 0
+        tapT = sBegin / stagesPerTap;
+        tapC = (sBegin - tapT * stagesPerTap) * BK;
+        tapR = tapT / p.kw;
+        tapS = tapT - tapR * p.kw;
+    }
+    auto tap_gather = [&]() __attribute__((always_inline)) {
+        const uint32_t voff = pixByte + 4u * (uint32_t)(tapR * p.W + tapS);
+        // the poison bit goes on last: the window origin of a border pixel is a negative (wrapped) offset,
+        // and adding a channel to an already poisoned offset could carry out of bit 31 again
+        uint32_t poison = 0;
+        if (MODE == IG_TAP_MASKED) {
+            const uint32_t word = tapT < 32 ? invLo : invHi;
+            poison = ((word >> (tapT & 31)) & 1u) << 31;
+        }
+        const uint32_t chan0 = (uint32_t)(tapC + grow0) * chanStep;
+#pragma unroll
+        for (int i = 0; i < B_LD; i++)
+            rb[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                        xres, (voff + (chan0 + (uint32_t)(i * TL::ROW_STEP) * chanStep)) | poison, 0, 0));
+        tapC += BK;
+        if (tapC == p.C) {
+            tapC = 0;
+            tapT++;
+            if (++tapS == p.kw) { tapS = 0; tapR++; }
+        }
+    };
     ag += (size_t)sBegin * aStage;
     ig_load_rows(ra, ag, aPass, SeqA());
     if (PW) {
         vg += (size_t)sBegin * vStage;
         ig_load_rows(rv, vg, vPass, SeqBV());
+    } else if (TAP) {
+        tap_gather();
     } else if (BUF) {
-        ig_gather_rows_buf<MODE == IG_BUF_MASKED>(rb, xres, pixByte, invLo, invHi, p.table, sBegin * BK + grow0, TL::ROW_STEP, p.kw, SeqB());
+        ig_gather_rows_buf<true>(rb, xres, pixByte, invLo, invHi, p.table, sBegin * BK + grow0, TL::ROW_STEP, p.kw, SeqB());
     } else {
         rbOk = ig_gather_rows<true>(rb, ximg, pixOff, maskR, maskS, p.table, sBegin * BK + grow0, TL::ROW_STEP, SeqB());
     }
@@ -270,7 +322,8 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
     auto load_stage = [&](const int s) __attribute__((always_inline)) {
         ig_load_rows(ra, ag + (size_t)(s - sBegin) * aStage, aPass, SeqA());
         if (PW) ig_load_rows(rv, vg + (size_t)(s - sBegin) * vStage, vPass, SeqBV());
-        else if (BUF) ig_gather_rows_buf<MODE == IG_BUF_MASKED>(rb, xres, pixByte, invLo, invHi, p.table, s * BK + grow0, TL::ROW_STEP, p.kw, SeqB());
+        else if (TAP) tap_gather();
+        else if (BUF) ig_gather_rows_buf<true>(rb, xres, pixByte, invLo, invHi, p.table, s * BK + grow0, TL::ROW_STEP, p.kw, SeqB());
         else rbOk = ig_gather_rows<true>(rb, ximg, pixOff, maskR, maskS, p.table, s * BK + grow0, TL::ROW_STEP, SeqB());
     };
     if (sBegin + 1 < sEnd) load_stage(sBegin + 1);
@@ -455,8 +508,10 @@ void launch(fc_context *ctx, IgemmParams &p) {
                         (p.C * p.kh * p.kw) % TL::BK_ == 0;
     // one 32-bit byte offset with bit 31 to spare reaches every element of the tensor
     const bool buffer = p.xBytes < (1l << 31);
+    const bool tapMajor = p.C % TL::BK_ == 0;      // the order fc_igemm_pack_filter laid the filter out in
     if (pointwise) igemm_conv_kernel<TL, IG_POINTWISE><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
-    else if (buffer && inside) igemm_conv_kernel<TL, IG_BUF_INSIDE><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
+    else if (buffer && tapMajor && inside) igemm_conv_kernel<TL, IG_TAP_INSIDE><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
+    else if (buffer && tapMajor && p.kh * p.kw <= 64) igemm_conv_kernel<TL, IG_TAP_MASKED><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
     else if (buffer && p.kh * p.kw <= 64) igemm_conv_kernel<TL, IG_BUF_MASKED><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);      // the taps of a window are one 64-bit mask
     else igemm_conv_kernel<TL, IG_GATHER><<<grid, dim3(TL::THREADS), 0, ctx->stream>>>(p);
 }
@@ -558,9 +613,12 @@ extern "C" int fc_igemm_pack_filter(fc_context *ctx, const fc_igemm_plan *plan, 
     const fc_conv_shape &s = plan->shape;
     const dim3 grid((plan->K_pad + 63) / 64, (plan->Kred_pad + 3) / 4);
     if (grid.y > 65535) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_igemm_pack_filter: reduction too long", hipSuccess);
+    fc_gemm_config cfg;
+    fc_igemm_get_config(plan->config, &cfg);
+    const int tapMajor = s.C % cfg.bk == 0 ? 1 : 0;      // must match the kernel's choice in launch()
     fc_stage_scope scope(ctx, FC_STAGE_FILTER_PACK);
     igemm_pack_filter_kernel<<<grid, dim3(256), 0, ctx->stream>>>(w_dev, Wp_dev, table_dev, s.K, s.C, s.kh, s.kw, s.H,
-                                                                 s.W, plan->Kred, plan->Kred_pad, plan->K_pad);
+                                                                 s.W, plan->Kred, plan->Kred_pad, plan->K_pad, tapMajor);
     FC_LAUNCH_CHECK(ctx, "igemm_pack_filter_kernel");
     return FC_OK;
 }
