@@ -65,7 +65,7 @@ def test_winograd_stage_by_stage(lib, shp, cfg):
 # -------------------------------------------------------- Winograd whole conv
 
 WINO_SHAPES = [
-    (1, 64, 56, 56, 64),       # BASELINE config 1
+    (1, 64, 56, 56, 64),       # the single-layer case the reference itself runs on a CPU: 64 -> 64 channels at 56x56
     (1, 1, 6, 6, 1), (1, 3, 7, 7, 7), (2, 64, 8, 8, 6), (1, 3, 13, 13, 5), (1, 64, 14, 14, 9),
     (1, 1, 28, 28, 3), (1, 3, 56, 56, 2), (2, 5, 9, 23, 11), (1, 4, 224, 224, 3), (1, 2, 112, 112, 5),
     (5, 7, 7, 7, 130), (32, 16, 14, 14, 16), (3, 130, 28, 28, 40),
@@ -306,7 +306,7 @@ def test_winograd_rejects_unsupported(lib):
 # -------------------------------------------------------------- implicit GEMM
 
 IGEMM_SHAPES = [
-    (1, 256, 56, 56, 256, 3, 3, 1, 1, 1),        # BASELINE config 2, layer A
+    (1, 256, 56, 56, 256, 3, 3, 1, 1, 1),        # the three im2col workload layers: A (3x3, 256 channels at 56x56)
     (1, 128, 56, 56, 256, 3, 3, 2, 2, 1),        # layer B
     (1, 256, 14, 14, 1024, 1, 1, 1, 1, 0),       # layer C
     (1, 3, 224, 224, 64, 7, 7, 2, 2, 3),         # ResNet-50 stem

@@ -44,7 +44,7 @@ def test_golden_vectors_match_reference_naive_layers():
 
 @pytest.mark.skipif(O.ref_lib() is None, reason="oracle/_ref not built (no reference checkout)")
 @pytest.mark.parametrize("shape", [
-    (1, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1),      # BASELINE config 1
+    (1, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1),      # the single-layer case the reference itself runs on a CPU: 64 -> 64 channels at 56x56
     (1, 16, 28, 28, 24, 3, 3, 1, 1, 1, 1, 1, 1),
 ])
 def test_live_reference_naive_3x3(shape):
