@@ -62,7 +62,7 @@ extern "C" int fc_init(int device, fc_context **out) {
     ctx->magic = FC_CTX_MAGIC;
     ctx->device = device;
     ctx->timing_mask = 0;
-    ctx->fused_lds_granted = ctx->onepass_lds_granted = false;
+    ctx->fused_lds_granted = ctx->onepass_lds_granted = ctx->smallc_lds_granted = false;
     ctx->capturing = false;
     ctx->stream = nullptr;
     ctx->probe_stream = nullptr;

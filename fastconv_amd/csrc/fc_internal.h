@@ -25,7 +25,7 @@ struct fc_context {
     double stage_ms[FC_STAGE_COUNT];
     long stage_launches[FC_STAGE_COUNT];
     // large dynamic LDS sizes are granted per kernel and per device, once per context
-    bool fused_lds_granted, onepass_lds_granted;
+    bool fused_lds_granted, onepass_lds_granted, smallc_lds_granted;
     bool capturing;         // between fc_graph_begin and fc_graph_end
     // shader-clock probe: its own stream and result buffer, created on first use
     hipStream_t probe_stream;
@@ -57,6 +57,12 @@ int fc_set_error(fc_context *ctx, int status, const char *what, hipError_t err);
 // implicit_gemm.hip: looks up the static workspace of this context's device (once per device)
 int fc_igemm_static_init(fc_context *ctx);
 bool fc_ctx_ok(const fc_context *ctx);
+// wino_smallc.hip: the single-kernel Winograd path of layers with at most four input channels.
+// Called by the fc_wino_*onepass* entry points after they have checked plan and pointers.
+bool fc_wino_smallc_applies(const fc_conv_shape *s);
+int fc_wino_smallc_filter_transform(fc_context *ctx, const fc_wino_plan *plan, const float *w_dev, float *U_dev);
+int fc_wino_smallc_conv(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev, const float *U_dev,
+                        const float *bias_dev, int relu, float *y_dev);
 
 // Brackets one kernel launch with events when timing is on.
 struct fc_stage_scope {

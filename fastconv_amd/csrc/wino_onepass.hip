@@ -350,6 +350,7 @@ extern "C" int fc_wino_onepass_filter_transform(fc_context *ctx, const fc_wino_p
                                                 float *U_dev) {
     const int rc = onepass_plan_check(ctx, plan, w_dev, U_dev);
     if (rc) return rc;
+    if (fc_wino_smallc_applies(&plan->shape)) return fc_wino_smallc_filter_transform(ctx, plan, w_dev, U_dev);
     const dim3 grid((plan->K_pad + 63) / 64, (plan->C_pad + 3) / 4);
     if (grid.y > 65535) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_onepass_filter_transform: too many channels", hipSuccess);
     fc_stage_scope scope(ctx, FC_STAGE_KERNEL_TRAN);
@@ -366,6 +367,7 @@ extern "C" int fc_wino_conv_onepass(fc_context *ctx, const fc_wino_plan *plan, c
     if (!y_dev) return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_conv_onepass: null output", hipSuccess);
     if (((uintptr_t)y_dev & 7) != 0 || ((uintptr_t)U_dev & 15) != 0 || ((uintptr_t)x_dev & 3) != 0)
         return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_conv_onepass: y must be 8-byte and U 16-byte aligned", hipSuccess);
+    if (fc_wino_smallc_applies(&plan->shape)) return fc_wino_smallc_conv(ctx, plan, x_dev, U_dev, bias_dev, relu, y_dev);
     if (!ctx->onepass_lds_granted) {
         if (ctx->capturing)
             return fc_set_error(ctx, FC_ERR_STATE, "fc_wino_conv_onepass: run this kernel once before recording a graph with it", hipSuccess);
@@ -391,6 +393,8 @@ extern "C" int fc_wino_conv_onepass(fc_context *ctx, const fc_wino_plan *plan, c
 
 extern "C" int fc_wino_prefer_onepass(const fc_conv_shape *s) {
     if (!fc_shape_ok(s) || s->kh != 3 || s->kw != 3 || s->sh != 1 || s->sw != 1 || s->W < 8) return 0;
+    // at most four channels: a kernel of its own on the vector ALUs, the fastest Winograd path at every batch
+    if (fc_wino_smallc_applies(s)) return 1;
     if (s->C < 16 || s->C > 64) return 0;
     // one 16-tile x 64-channel block per workgroup, one workgroup per CU at a time: the layer must
     // bring a few blocks per CU (batch 1 layers do not).  Measured crossover against the staged

@@ -205,6 +205,29 @@ def test_winograd_single_kernel_against_oracle(lib, shp, pads):
     assert O.max_rel_err(y2, O.naive_conv_f64(s, x, w)) <= TOL_WINO
 
 
+@pytest.mark.parametrize("shp,pads", [
+    ((1, 1, 20, 20, 1), {}), ((2, 2, 31, 40, 17), {}), ((3, 3, 45, 45, 64), {}), ((2, 3, 44, 46, 70), {}),
+    ((1, 4, 64, 64, 130), {}), ((2, 4, 23, 24, 9), {"pt": 0, "pb": 2, "pl": 2, "pr": 0}), ((7, 3, 32, 32, 32), {}),
+    ((1, 3, 100, 372, 5), {}), ((8, 3, 384, 384, 6), {}), ((2, 3, 8, 8, 3), {"pt": 2, "pl": 0}),
+])
+def test_winograd_small_channel_kernel(lib, shp, pads):
+    """Layers with at most four input channels run through a kernel of their own behind the
+    single-kernel entry points: every channel count, even and odd output widths (rows stored
+    through LDS or every lane its own block), output channels that do not fill a wavefront's
+    share, tile counts off the 62 / 64 tiles of a workgroup, 16 and 64 channels per workgroup."""
+    s = O.shape(*shp, **pads)
+    assert lib.wino_prefer_onepass(cshape(s))
+    x, w = O.make_inputs(s, seed=shp[1] + 71)
+    bias = O.rng_uniform(9, (s.K,))
+    announce("small-channel winograd", shp, pads)
+    y = lib.winograd_conv_onepass(cshape(s), x, w, bias=bias, relu=True)
+    truth = np.maximum(O.naive_conv_f64(s, x, w, bias), 0.0)
+    assert y.shape == truth.shape
+    assert O.max_rel_err(y, truth) <= TOL_WINO
+    y2 = lib.winograd_conv_onepass(cshape(s), x, w)
+    assert O.max_rel_err(y2, O.naive_conv_f64(s, x, w)) <= TOL_WINO
+
+
 def test_winograd_single_kernel_full_size_layers(lib):
     for (N, C, H, K) in [(32, 3, 224, 64), (32, 64, 112, 128), (8, 64, 224, 64)]:
         s = O.shape(N, C, H, H, K)
