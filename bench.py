@@ -71,6 +71,7 @@ WORKLOADS = {
     "resnet50_3x3_b1": (_w(RESNET50_3X3), 1, "winograd", "ResNet-50 3x3 s1 convs, Winograd F(6,3), batch 1"),
     "im2col_abc_b1": (IM2COL_ABC, 1, "im2col", "3x3 256@56, 3x3 s2 128->256@56, 1x1 256->1024@14 through the implicit GEMM, batch 1"),
     "cfg1": (_w([(64, 64, 56, 1)]), 1, "winograd", "single 3x3 conv 64->64 @56, batch 1"),
+    "conv3_224_b32": (_w([(3, 64, 224, 1)]), 32, "winograd", "single 3x3 conv 3->64 @224, batch 32 (VGG-16 layer 1)"),
     "conv64_224_b32": (_w([(64, 64, 224, 1)]), 32, "winograd", "single 3x3 conv 64->64 @224, batch 32 (VGG-16 layer 2)"),
     "conv256_56_b32": (_w([(256, 256, 56, 1)]), 32, "winograd", "single 3x3 conv 256->256 @56, batch 32 (VGG-16 layers 6-7)"),
     "conv512_28_b32": (_w([(512, 512, 28, 1)]), 32, "winograd", "single 3x3 conv 512->512 @28, batch 32 (VGG-16 layers 9-10)"),
@@ -555,6 +556,8 @@ def run_workload(name, steps, warmup, o, detail=True, offline_filter=None):
             "frac": round(oflops * k / (onepass_stage[0] * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 4),
             "launches": onepass_stage[1], "avg_launch_ms": round(onepass_stage[0] / onepass_stage[1], 5),
             "hbm_gbs": round(gbs, 1)}
+        if any(l.C <= 4 for l in ol):
+            transforms["single_kernel_conv"]["note"] = "includes the launches of the small-channel kernel (no per-layer pass in this run)"
 
     igemm_events = None
     if igemm_stage[1] > 0:
@@ -699,6 +702,38 @@ def run_workload(name, steps, warmup, o, detail=True, offline_filter=None):
                 row["faster_class"] = "zc" if cands["zc"]["ms"] <= cands["blocked"]["ms"] else "blocked"
         for lay, (pipe, plan, U, ib, bp) in zip(layers, saved):
             lay.pipe, lay.plan, lay.U, lay.img_block, lay.block_plans = pipe, plan, U, ib, bp
+
+    # Two kernels answer the single-kernel calls: the MFMA one and, for layers of at most four input
+    # channels, one on the vector ALUs that is bound by the stores of y.  The library books both under
+    # one stage, so the two lines are taken from the per-layer pass, which times every layer by itself.
+    op_rows = [(l, r) for l, r in zip(layers, per_layer) if r.get("pipeline") == "onepass"]
+    if op_rows:
+        def kernel_ms(rows):
+            return sum(r["stage_ms"]["gemm"] * l.repeats for l, r in rows)
+        big = [(l, r) for l, r in op_rows if l.C > 4]
+        small = [(l, r) for l, r in op_rows if l.C <= 4]
+        was_roofline = roofline.get("kernel") == "wino_onepass_kernel"
+        transforms.pop("single_kernel_conv", None)
+        if big:
+            ms = kernel_ms(big)
+            fl = sum(l.algorithmic()["gemm_flops"] * l.repeats for l, _ in big)
+            by = sum((4.0 * l.N * l.C * l.H * l.H + 256.0 * l.K * l.C + 4.0 * l.N * l.K * l.H * l.H) * l.repeats for l, _ in big)
+            transforms["single_kernel_conv"] = {
+                "kernel": "wino_onepass_kernel", "bound": "mfma", "achieved": round(fl / (ms * 1e-3) / 1e12, 2),
+                "peak": PEAK_MFMA_F32_TFLOPS, "unit": "TFLOP/s", "frac": round(fl / (ms * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 4),
+                "launches_per_step": sum(l.repeats for l, _ in big), "ms_per_step": round(ms, 4),
+                "hbm_gbs": round(by / (ms * 1e-3) / 1e9, 1)}
+        if small:
+            ms = kernel_ms(small)
+            by = sum((4.0 * l.N * l.C * l.H * l.H + 1024.0 * l.K + 4.0 * l.N * l.K * l.H * l.H) * l.repeats for l, _ in small)
+            transforms["small_channel_conv"] = {
+                "kernel": "wino_smallc_kernel", "bound": "hbm", "achieved": round(by / (ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
+                "unit": "GB/s", "frac": round(by / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                "launches_per_step": sum(l.repeats for l, _ in small), "ms_per_step": round(ms, 4),
+                "note": "x, the transformed filter and y once; vector ALUs only"}
+        if was_roofline:
+            src = transforms.get("single_kernel_conv") or transforms["small_channel_conv"]
+            roofline = dict(src, traffic=None)
 
     roofline["events"] = ("inside the timed region" if stage_events in ("gemm", "all") and not o.graph
                           else "in the untimed steps after it")

@@ -337,8 +337,8 @@ extern "C" int fc_wino_make_plan(const fc_conv_shape *s, int gemm_config, fc_win
 // stride-1 layer of VGG-16 and ResNet-50 at batch 1 and 32): Winograd wins on every layer with at
 // least 1.85 GFLOP of direct-convolution work and 16 or more input channels (by 1.25x to 3.9x), the
 // implicit GEMM on every layer of 0.92 GFLOP or less (batch-1 layers: one launch against three, and no
-// 64x larger transformed filter to write and read) and on the 3-channel first layer (1.9x to 2.2x:
-// the 64 planes of M carry no reuse over 3 channels).
+// 64x larger transformed filter to write and read); on the 3-channel first layer the two are level at
+// batch 32 (both bound by the stores of the output) and the implicit GEMM is 2.1x ahead at batch 1.
 extern "C" int fc_prefer_winograd(const fc_conv_shape *s) {
     if (!fc_shape_ok(s) || s->kh != 3 || s->kw != 3 || s->sh != 1 || s->sw != 1) return 0;
     const int OH = fc_out_dim(s->H, s->pt, s->pb, 3, 1), OW = fc_out_dim(s->W, s->pl, s->pr, 3, 1);

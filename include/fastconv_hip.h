@@ -259,6 +259,10 @@ int fc_wino_forward_fused(fc_context *ctx, const fc_wino_plan *plan, const float
  * fc_wino_onepass_filter_transform writes it and
  * only fc_wino_conv_onepass reads it.  The stage calls above reject such a plan.
  * Images narrower than 8 columns are not supported (FC_ERR_UNSUPPORTED): use the staged calls.
+ * Layers with at most four input channels (and an input of at most 2 GiB) run through a kernel
+ * of their own on the vector ALUs behind the same three calls (the products are too few for the
+ * matrix cores to matter and the layer is bound by the stores of y); their transformed filter
+ * is laid out [K_pad][8][8][4] in the same buffer.
  * The GPU reading of the reference's blocked pipeline taken to its end: there one block of
  * tiles goes through input transform, TensorGEMM and output transform out of block-local
  * scratch (winoF63/winoF63.cpp:1574-1737); here the block-local scratch is LDS and registers. */
@@ -281,7 +285,7 @@ int fc_wino_forward_onepass(fc_context *ctx, const fc_wino_plan *plan, const flo
  * layer (measured on MI355X: 16 to 64 input channels, where the products are cheap next to
  * moving V and M through HBM, the image at least 8 columns wide, and at least 512 blocks of
  * 16 tiles x 64 output channels -- 192 when one block covers all output channels -- i.e. not
- * at batch 1). */
+ * at batch 1; and every layer with at most four input channels, at any batch). */
 int fc_wino_prefer_onepass(const fc_conv_shape *shape);
 
 /* All stages back to back: what winoF63_v1_single (winoF63ZC/winoF63ZC.h:5-6)
