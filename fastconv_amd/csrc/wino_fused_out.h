@@ -64,18 +64,19 @@ __device__ __forceinline__ void fused_output_transform(const FusedOut &p, const 
             const uint32_t th = fc_div(r, p.divTW), tw = r - th * p.tW;
             const int rows = min(6, p.OH - (int)th * 6), cols = min(6, p.OW - (int)tw * 6);
             const float bias = p.bias ? p.bias[k] : 0.f;
+            const float floorv = p.relu ? 0.f : -__builtin_inff();
             float *dst = p.y + (((size_t)n * p.K + k) * p.OH + (size_t)th * 6) * p.OW + tw * 6;
             const bool pairs = cols == 6 && (p.OW & 1) == 0;    // 8-byte aligned row segments
 #pragma unroll
             for (int i = 0; i < 6; i++) {
+                // the bias goes in with element 1 (at6 adds it, as m1 + m2 or m1 - m2, to each output once):
+                // the same order of additions as in the staged output transform, whose results this kernel equals bit for bit
+                const float rowv[8] = {tmp[i][0], tmp[i][1] + bias, tmp[i][2], tmp[i][3], tmp[i][4], tmp[i][5], tmp[i][6], tmp[i][7]};
                 float sres[6];
-                at6(tmp[i], sres);
+                at6(rowv, sres);
                 if (i < rows) {
 #pragma unroll
-                    for (int jj = 0; jj < 6; jj++) {
-                        sres[jj] += bias;
-                        if (p.relu) sres[jj] = fmaxf(sres[jj], 0.f);
-                    }
+                    for (int jj = 0; jj < 6; jj++) sres[jj] = fmaxf(sres[jj], floorv);
                     float *drow = dst + (size_t)i * p.OW;
                     if (pairs) {
 #pragma unroll

@@ -9,13 +9,20 @@
 
 namespace {
 
+// Uniform base pointer + 32-bit byte offset of the lane: the address form that costs no vector
+// instruction (the base lives in scalar registers, the offset is one register shared by all the
+// loads or stores of the lane).
 // M is read exactly once, by the output transform: loaded with the non-temporal hint it does not
 // displace what the caches hold for the kernels around it (measured on the batch-32 VGG-16 layers:
 // the output transform 6 % shorter over the stack, 14 % on 128 -> 128 channels at 112x112).  The
 // same hint on the stores of V makes the input transform 40 % faster when it runs by itself, and
-// slower inside the pipeline: the GEMM that follows is MFMA-bound and hides the write-back of V,
-// which it then finds in the last-level cache; with the hint the transform pays for the write itself.
-__device__ __forceinline__ float load_m(const float *p) { return __builtin_nontemporal_load(p); }
+// slower inside the pipeline.
+__device__ __forceinline__ float load_m_at(const float *base, uint32_t byteOff) {
+    return __builtin_nontemporal_load(reinterpret_cast<const float *>(reinterpret_cast<const char *>(base) + byteOff));
+}
+__device__ __forceinline__ void store_at(float *base, uint32_t byteOff, float v) {
+    *reinterpret_cast<float *>(reinterpret_cast<char *>(base) + byteOff) = v;
+}
 
 // ---------------------------------------------------------------- filter
 
@@ -32,8 +39,9 @@ __device__ __forceinline__ void filter_transform_block(const FilterTParams &q, i
     const float *__restrict__ w = q.w;
     float *__restrict__ U = q.U;
     const int K = q.K, C = q.C, K_pad = q.K_pad, C_pad = q.C_pad;
-    const int k = bx * 64 + (threadIdx.x & 63);
-    const int c = by * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int k = bx * 64 + lane;
+    const int c = by * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (k >= K_pad || c >= C_pad) return;
     float g[3][3];
     if (k < K && c < C) {
@@ -55,13 +63,17 @@ __device__ __forceinline__ void filter_transform_block(const FilterTParams &q, i
         for (int i = 0; i < 8; i++) t[i][j] = o[i];
     }
     const size_t plane = (size_t)C_pad * K_pad;
-    float *dst = U + (size_t)c * K_pad + k;
+    float *pf = U + (size_t)c * K_pad + bx * 64;       // uniform; the lane adds 4 * lane
+    const uint32_t laneOff = (uint32_t)lane * 4u;
 #pragma unroll
     for (int i = 0; i < 8; i++) {
         float o[8];
         g8(t[i], o);
 #pragma unroll
-        for (int j = 0; j < 8; j++) dst[(size_t)(i * 8 + j) * plane] = o[j];
+        for (int j = 0; j < 8; j++) {
+            store_at(pf, laneOff, o[j]);
+            pf += plane;
+        }
     }
 }
 
@@ -82,6 +94,7 @@ struct InTParams {
     int N, C, H, W, pad_t, pad_l;
     int tH, tW;
     long T;          // real tiles; tiles in [T, T_pad) are written as zeros
+    unsigned xBytes; // size of x when it is at most 2 GiB (the buffer path), else unused
     int C_pad;
     long T_pad;
     int LW;          // 6*tW + 2: columns of a band as its tiles see it, padding columns included
@@ -94,7 +107,12 @@ struct InTParams {
 // row-contiguous.  Pass 2 applies B along the rows out of LDS: a thread owns one
 // tile and 8*TPB/256 of its 8 rows, and stores to the frequency planes with lanes
 // on consecutive tiles.
-template <int TPB, int ITEMS>
+// BUF: x is read through a buffer resource with 32-bit byte offsets; an element outside the image
+// (or a column this block does not need) gets an offset with bit 31 set, which is past the end of
+// x, and the hardware returns zero: no branch and no 64-bit address per load.  Inputs of more than
+// 2 GiB take the pointer path.  The plane stores of pass 2 use a scalar base per frequency and one
+// 32-bit lane offset (the kernel spent half of its vector instructions on addresses before).
+template <int TPB, int ITEMS, bool BUF>
 __device__ __forceinline__ void input_transform_block(const InTParams &p, int bx, int c, float *lds) {
     const int tid = threadIdx.x;
     const size_t plane = (size_t)p.C_pad * p.T_pad;
@@ -111,27 +129,53 @@ __device__ __forceinline__ void input_transform_block(const InTParams &p, int bx
         const int items = NB * p.LW;
         float d[ITEMS][8];
         int dstOff[ITEMS];
+        if (BUF) {
+            __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.x), 0, (int)p.xBytes, 0x00020000);
+            const uint32_t chanOff = (uint32_t)c * (uint32_t)(p.H * p.W);
+            const uint32_t imgStride = (uint32_t)p.C * (uint32_t)(p.H * p.W);
 #pragma unroll
-        for (int it = 0; it < ITEMS; it++) {
-            const int e = tid + it * 256;
-            dstOff[it] = -1;
-#pragma unroll
-            for (int i = 0; i < 8; i++) d[it][i] = 0.f;
-            if (e < items) {
+            for (int it = 0; it < ITEMS; it++) {
+                const int e = tid + it * 256;
                 const int j = fc_div(e, p.divLW), lx = e - j * p.LW;
                 // columns this block needs of band j
                 const int lxA = (j == 0) ? tw0 * 6 : 0, lxB = (j == NB - 1) ? twL * 6 + 8 : p.LW;
-                if (lx >= lxA && lx < lxB) {
-                    dstOff[it] = j * 8 * p.LW + lx;
-                    const uint32_t gb = gb0 + j;
-                    const uint32_t n = fc_div(gb, p.divTH), th = gb - n * p.tH;
-                    const int gx = lx - p.pad_l, gy0 = (int)th * 6 - p.pad_t;
-                    if (gx >= 0 && gx < p.W) {
-                        const float *src = p.x + (((size_t)n * p.C + c) * p.H) * p.W + gx;
+                const bool need = e < items && lx >= lxA && lx < lxB;
+                dstOff[it] = need ? j * 8 * p.LW + lx : -1;
+                const uint32_t gb = gb0 + j;
+                const uint32_t n = fc_div(gb, p.divTH), th = gb - n * p.tH;
+                const int gx = lx - p.pad_l, gy0 = (int)th * 6 - p.pad_t;
+                const bool colIn = need && (uint32_t)gx < (uint32_t)p.W;
+                // byte offset of row gy0 (possibly above the image: then only rows that are inside are used)
+                const uint32_t off0 = (n * imgStride + chanOff + (uint32_t)(gy0 * p.W + gx)) * 4u;
 #pragma unroll
-                        for (int i = 0; i < 8; i++) {
-                            const int gy = gy0 + i;
-                            if (gy >= 0 && gy < p.H) d[it][i] = src[(long)gy * p.W];
+                for (int i = 0; i < 8; i++) {
+                    const bool in = colIn && (uint32_t)(gy0 + i) < (uint32_t)p.H;
+                    const uint32_t off = in ? off0 + (uint32_t)(i * p.W) * 4u : 0x80000000u;
+                    d[it][i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xres, (int)off, 0, 0));
+                }
+            }
+        } else {
+#pragma unroll
+            for (int it = 0; it < ITEMS; it++) {
+                const int e = tid + it * 256;
+                dstOff[it] = -1;
+#pragma unroll
+                for (int i = 0; i < 8; i++) d[it][i] = 0.f;
+                if (e < items) {
+                    const int j = fc_div(e, p.divLW), lx = e - j * p.LW;
+                    const int lxA = (j == 0) ? tw0 * 6 : 0, lxB = (j == NB - 1) ? twL * 6 + 8 : p.LW;
+                    if (lx >= lxA && lx < lxB) {
+                        dstOff[it] = j * 8 * p.LW + lx;
+                        const uint32_t gb = gb0 + j;
+                        const uint32_t n = fc_div(gb, p.divTH), th = gb - n * p.tH;
+                        const int gx = lx - p.pad_l, gy0 = (int)th * 6 - p.pad_t;
+                        if (gx >= 0 && gx < p.W) {
+                            const float *src = p.x + (((size_t)n * p.C + c) * p.H) * p.W + gx;
+#pragma unroll
+                            for (int i = 0; i < 8; i++) {
+                                const int gy = gy0 + i;
+                                if (gy >= 0 && gy < p.H) d[it][i] = src[(long)gy * p.W];
+                            }
                         }
                     }
                 }
@@ -151,44 +195,52 @@ __device__ __forceinline__ void input_transform_block(const InTParams &p, int bx
     __syncthreads();
 
     constexpr int IPT = 8 * TPB / 256;     // rows of the 8x8 tile per thread
-    const int tl = tid % TPB, ig = tid / TPB;
+    const int tl = tid % TPB;
+    // rows ig*IPT .. +IPT-1 of the tile: the same for a whole wavefront when TPB is a multiple of 64
+    const int igLane = tid / TPB;
+    const int ig = TPB >= 64 ? __builtin_amdgcn_readfirstlane(igLane) : igLane;
     const uint32_t t = t0 + tl;
-    float *dst = p.V + (size_t)c * p.T_pad + t;
+    // plane f of this block starts at V + f * plane + c * T_pad + t0; the lane adds 4 * tl
+    // (with 32 tiles per block the two halves of a wavefront are on different planes: a pointer per lane)
+    float *pf = p.V + (size_t)(ig * IPT * 8) * plane + (size_t)c * p.T_pad + t0;
+    const uint32_t laneOff = (uint32_t)tl * 4u;
     if (c < p.C && t < (uint32_t)p.T) {
         const uint32_t gb = fc_div(t, p.divTW);
         const int q = t - gb * p.tW, j = gb - gb0;
+        const float *rows = lds + (j * 8 + ig * IPT) * p.LW + q * 6;
 #pragma unroll
         for (int ii = 0; ii < IPT; ii++) {
-            const int i = ig * IPT + ii;
-            const float *row = lds + ((size_t)j * 8 + i) * p.LW + q * 6;
+            const float *row = rows + ii * p.LW;
             float d[8], o[8];
 #pragma unroll
             for (int jj = 0; jj < 8; jj++) d[jj] = row[jj];
             bt8(d, o);
 #pragma unroll
-            for (int jj = 0; jj < 8; jj++) dst[(size_t)(i * 8 + jj) * plane] = o[jj];
+            for (int jj = 0; jj < 8; jj++) {
+                store_at(pf, laneOff, o[jj]);
+                pf += plane;       // stepped, not multiplied: a 64-bit product would be made with vector instructions
+            }
         }
     } else {
         // padding channel or padding tile: the GEMM reads it, so it must be zero
 #pragma unroll
-        for (int ii = 0; ii < IPT; ii++) {
-            const int i = ig * IPT + ii;
-#pragma unroll
-            for (int jj = 0; jj < 8; jj++) dst[(size_t)(i * 8 + jj) * plane] = 0.f;
+        for (int ii = 0; ii < IPT * 8; ii++) {
+            store_at(pf, laneOff, 0.f);
+            pf += plane;
         }
     }
 }
 
-template <int TPB, int ITEMS>
+template <int TPB, int ITEMS, bool BUF>
 __global__ __launch_bounds__(256) void wino_input_transform_kernel(const InTParams p) {
     extern __shared__ float lds[];   // [bands][8][LW]
-    input_transform_block<TPB, ITEMS>(p, blockIdx.x, blockIdx.y, lds);
+    input_transform_block<TPB, ITEMS, BUF>(p, blockIdx.x, blockIdx.y, lds);
 }
 
 // Filter and input transform in one launch (the filter transform of a layer is a short
 // kernel: launched by itself it costs a launch and a drain of the whole chip per layer).
 // The first nFilter workgroups transform the filter, the others the input.
-template <int TPB, int ITEMS>
+template <int TPB, int ITEMS, bool BUF>
 __global__ __launch_bounds__(256) void wino_filter_input_transform_kernel(const FilterTParams q, const InTParams p,
                                                                           int filterGridX, int nFilter, int inputGridX) {
     extern __shared__ float lds[];
@@ -198,7 +250,7 @@ __global__ __launch_bounds__(256) void wino_filter_input_transform_kernel(const 
         filter_transform_block(q, b - by * filterGridX, by);
     } else {
         const int i = b - nFilter, c = i / inputGridX;
-        input_transform_block<TPB, ITEMS>(p, i - c * inputGridX, c, lds);
+        input_transform_block<TPB, ITEMS, BUF>(p, i - c * inputGridX, c, lds);
     }
 }
 
@@ -221,10 +273,14 @@ struct OutTParams {
 // laid into LDS as the image rows they cover ([band][6][OW]) and copied out band
 // by band: a band the block covers completely is one contiguous run of rows*OW
 // floats, a partly covered band (first or last of the range) is one run per row.
+// Everything that does not depend on the lane (plane bases, band geometry of the
+// copy loop) is kept in scalar registers: the kernel spends a quarter of its
+// vector instructions on addresses otherwise.
 template <int TPB>
 __global__ __launch_bounds__(TPB) void wino_output_transform_kernel(const OutTParams p) {
     extern __shared__ __attribute__((aligned(16))) float lds[];   // [bands][6][OW]
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int k = blockIdx.y;
     const uint32_t t0 = blockIdx.x * TPB;
     if (t0 >= (uint32_t)p.T) return;
@@ -239,10 +295,15 @@ __global__ __launch_bounds__(TPB) void wino_output_transform_kernel(const OutTPa
         const uint32_t gb = fc_div(t, p.divTW);
         const int q = t - gb * p.tW, j = gb - gb0;
         const size_t plane = (size_t)p.K_pad * p.T_pad;
-        const float *src = p.M + (size_t)k * p.T_pad + t;
+        const float *src = p.M + (size_t)k * p.T_pad + t0;      // uniform
+        const uint32_t laneOff = (uint32_t)tid * 4u;
         float m[8][8];
+        const float *pf = src;      // stepped, not multiplied: a 64-bit product would be made with vector instructions
 #pragma unroll
-        for (int f = 0; f < 64; f++) m[f >> 3][f & 7] = load_m(src + (size_t)f * plane);
+        for (int f = 0; f < 64; f++) {
+            m[f >> 3][f & 7] = load_m_at(pf, laneOff);
+            pf += plane;
+        }
         float tmp[6][8];
 #pragma unroll
         for (int jj = 0; jj < 8; jj++) {
@@ -253,17 +314,25 @@ __global__ __launch_bounds__(TPB) void wino_output_transform_kernel(const OutTPa
             for (int i = 0; i < 6; i++) tmp[i][jj] = s[i];
         }
         const float b = p.bias ? p.bias[k] : 0.f;
-        float *img = lds + (size_t)j * bandElems + q * 6;
+        const float floorv = p.relu ? 0.f : -__builtin_inff();
+        float *img = lds + j * bandElems + q * 6;
         const int colsLeft = p.OW - q * 6;      // columns of this tile inside the image
 #pragma unroll
         for (int i = 0; i < 6; i++) {
+            // the bias goes in with element 1: at6 adds it (as m1 + m2 or m1 - m2) to each of its six outputs once
+            const float row[8] = {tmp[i][0], tmp[i][1] + b, tmp[i][2], tmp[i][3], tmp[i][4], tmp[i][5], tmp[i][6], tmp[i][7]};
             float s[6];
-            at6(tmp[i], s);
+            at6(row, s);
 #pragma unroll
-            for (int jj = 0; jj < 6; jj++) {
-                float v = s[jj] + b;
-                if (p.relu) v = fmaxf(v, 0.f);
-                if (jj < colsLeft) img[i * p.OW + jj] = v;
+            for (int jj = 0; jj < 6; jj++) s[jj] = fmaxf(s[jj], floorv);
+            float *dstl = img + i * p.OW;
+            if (colsLeft >= 6) {
+#pragma unroll
+                for (int jj = 0; jj < 6; jj++) dstl[jj] = s[jj];
+            } else {
+#pragma unroll
+                for (int jj = 0; jj < 6; jj++)
+                    if (jj < colsLeft) dstl[jj] = s[jj];
             }
         }
     }
@@ -271,27 +340,28 @@ __global__ __launch_bounds__(TPB) void wino_output_transform_kernel(const OutTPa
 
     constexpr int WAVES = TPB / 64;
     const bool vec4 = (p.OW & 3) == 0;
-    for (int j = wave; j < NB; j += WAVES) {
+    const size_t chan = (size_t)p.OH * p.OW;
+    for (int j = wave; j < NB; j += WAVES) {       // j and everything derived from it is uniform
         const uint32_t gb = gb0 + j;
         const uint32_t n = fc_div(gb, p.divTH), th = gb - n * p.tH;
         const int rows = min(6, p.OH - (int)th * 6);
         const int xA = (j == 0) ? tw0 * 6 : 0;
         const int xB = min((j == NB - 1) ? (twL + 1) * 6 : p.tW * 6, p.OW);
-        float *dst = p.y + (((size_t)n * p.K + k) * p.OH + (size_t)th * 6) * p.OW;
-        const float *src = lds + (size_t)j * bandElems;
+        float *dst = p.y + ((size_t)n * p.K + k) * chan + (size_t)th * 6 * p.OW;
+        const float *src = lds + j * bandElems;
         if (xA == 0 && xB == p.OW) {
             const int len = rows * p.OW;
             if (vec4) {
                 typedef float vec4 __attribute__((ext_vector_type(4)));
-                const vec4 *s4 = reinterpret_cast<const vec4 *>(src);
-                vec4 *d4 = reinterpret_cast<vec4 *>(dst);
-                for (int e = lane; e < len / 4; e += 64) d4[e] = s4[e];
+                for (int e = lane; e < len / 4; e += 64)
+                    *reinterpret_cast<vec4 *>(reinterpret_cast<char *>(dst) + (uint32_t)e * 16u) =
+                        *reinterpret_cast<const vec4 *>(reinterpret_cast<const char *>(src) + (uint32_t)e * 16u);
             } else {
-                for (int e = lane; e < len; e += 64) dst[e] = src[e];
+                for (int e = lane; e < len; e += 64) store_at(dst, (uint32_t)e * 4u, src[e]);
             }
         } else {
             for (int i = 0; i < rows; i++)
-                for (int x = xA + lane; x < xB; x += 64) dst[i * p.OW + x] = src[i * p.OW + x];
+                for (int x = xA + lane; x < xB; x += 64) store_at(dst + i * p.OW, (uint32_t)x * 4u, src[i * p.OW + x]);
         }
     }
 }
@@ -411,21 +481,26 @@ static int launch_input_transform(fc_context *ctx, const fc_wino_plan *plan, con
     const long nFilter = q ? (long)filterGridX * ((plan->C_pad + 3) / 4) : 0;
     const long total = nFilter + (long)grid.x * grid.y;
     if (total >= (1l << 31)) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_input_transform: grid too large", hipSuccess);
+    const size_t xBytes = sizeof(float) * s.N * s.C * s.H * s.W;
+    const bool useBuf = xBytes <= ((size_t)1 << 31);
+    p.xBytes = useBuf ? (unsigned)xBytes : 0u;
     fc_stage_scope scope(ctx, FC_STAGE_INPUT_TRAN);
-#define FC_LAUNCH_ONE(TPB_, ITEMS_)                                                                                      \
+#define FC_LAUNCH_ONE(TPB_, ITEMS_, BUF_)                                                                                \
     do {                                                                                                                 \
         if (q)                                                                                                           \
-            wino_filter_input_transform_kernel<TPB_, ITEMS_><<<dim3((unsigned)total), dim3(256), ldsBytes, ctx->stream>>>( \
+            wino_filter_input_transform_kernel<TPB_, ITEMS_, BUF_><<<dim3((unsigned)total), dim3(256), ldsBytes, ctx->stream>>>( \
                 *q, p, filterGridX, (int)nFilter, (int)grid.x);                                                          \
         else                                                                                                             \
-            wino_input_transform_kernel<TPB_, ITEMS_><<<grid, dim3(256), ldsBytes, ctx->stream>>>(p);                    \
+            wino_input_transform_kernel<TPB_, ITEMS_, BUF_><<<grid, dim3(256), ldsBytes, ctx->stream>>>(p);              \
     } while (0)
-#define FC_LAUNCH_INT(TPB_)                                  \
-    do {                                                     \
-        if (itemsPerThread <= 2) FC_LAUNCH_ONE(TPB_, 2);     \
-        else if (itemsPerThread <= 4) FC_LAUNCH_ONE(TPB_, 4); \
-        else if (itemsPerThread <= 6) FC_LAUNCH_ONE(TPB_, 6); \
-        else FC_LAUNCH_ONE(TPB_, 8);                         \
+    // the pointer path (inputs of more than 2 GiB) is built for 8 columns per thread only
+#define FC_LAUNCH_INT(TPB_)                                        \
+    do {                                                           \
+        if (!useBuf) FC_LAUNCH_ONE(TPB_, 8, false);                \
+        else if (itemsPerThread <= 2) FC_LAUNCH_ONE(TPB_, 2, true); \
+        else if (itemsPerThread <= 4) FC_LAUNCH_ONE(TPB_, 4, true); \
+        else if (itemsPerThread <= 6) FC_LAUNCH_ONE(TPB_, 6, true); \
+        else FC_LAUNCH_ONE(TPB_, 8, true);                         \
     } while (0)
     if (tpb == 128) FC_LAUNCH_INT(128);
     else if (tpb == 64) FC_LAUNCH_INT(64);
