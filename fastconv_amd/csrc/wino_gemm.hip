@@ -17,10 +17,28 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 // Copy passes written as pack expansions, so that every register-array index is a
 // literal constant: with a loop index the arrays are not promoted to registers
 // and the tile makes a round trip through scratch memory.
+// `base` is the same for the whole workgroup (it stays in scalar registers); a lane adds its
+// 32-bit byte offset: no vector instruction goes into the addresses.
+// A pointer that is the same for every lane, pinned to scalar registers: without the pin the
+// compiler turns a uniform base that advances in a loop into a 64-bit pointer per lane and pays
+// a vector add per access.
+template <class T>
+__device__ __forceinline__ T *uniform_ptr(T *p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    // through a global-memory pointer type: rebuilt from an integer the pointer would otherwise be a generic one
+    typedef __attribute__((address_space(1))) T GlobalT;
+    return (T *)reinterpret_cast<GlobalT *>(((uint64_t)hi << 32) | lo);
+}
+
 template <int... I>
-__device__ __forceinline__ void load_rows(floatx4 (&r)[sizeof...(I)], const float *p, size_t rowStride,
+__device__ __forceinline__ void load_rows(floatx4 (&r)[sizeof...(I)], const float *base, uint32_t laneOff, size_t rowStride,
                                           std::integer_sequence<int, I...>) {
-    ((r[I] = *reinterpret_cast<const floatx4 *>(p + (size_t)I * rowStride)), ...);
+    // row after row by addition: pinned operands keep the sums in the scalar unit.  The empty asm keeps the widening of
+    // the lane offset next to the loads (hoisted out of a loop it turns each address into a 64-bit vector sum)
+    asm volatile("" : "+v"(laneOff));
+    const float *b = uniform_ptr(base);
+    ((r[I] = *reinterpret_cast<const floatx4 *>(reinterpret_cast<const char *>(b) + laneOff), b = uniform_ptr(b + rowStride)), ...);
 }
 template <int... I>
 __device__ __forceinline__ void store_rows(float *lds, const floatx4 (&r)[sizeof...(I)], int rowStride,
@@ -50,7 +68,7 @@ struct GemmTile {
     static constexpr int A_ROWS = THREADS * 4 / BM, B_ROWS = THREADS * 4 / BN;   // tile rows per copy pass
     static constexpr int LDS_BYTES = 2 * BK * (BM + BN) * 4;
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be whole 32x32 MFMA blocks");
-    static_assert(BK % 2 == 0, "32x32x2 MFMA consumes two reduction steps");
+    static_assert(BK % 4 == 0, "fragments are fetched for two 32x32x2 MFMA steps at a time");
     static_assert(A_VEC % THREADS == 0 && B_VEC % THREADS == 0, "every thread copies the same number of float4");
     static_assert(A_LD >= 1 && B_LD >= 1, "tile smaller than one copy pass");
 };
@@ -66,14 +84,17 @@ __device__ __forceinline__ void gemm_tile(const float *__restrict__ U, const flo
     // LDS: A stages 0 and 1, then B stages 0 and 1
     float *const As0 = smem, *const Bs0 = smem + 2 * BK * BM;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm0 = (wave / TL::WGN_) * TL::WM, wn0 = (wave % TL::WGN_) * TL::WN;
 
     // this thread's float4 of each copy pass: row r0 + i*ROWS, column c4
     const int arow = tid / (BM / 4), acol = (tid % (BM / 4)) * 4;
     const int brow = tid / (BN / 4), bcol = (tid % (BN / 4)) * 4;
-    const float *ag = U + ((size_t)f * C_pad + arow) * K_pad + (size_t)kb * BM + acol;
-    const float *bg = V + ((size_t)f * C_pad + brow) * T_pad + (size_t)tb * BN + bcol;
+    // global tiles: a uniform base per operand and stage, and one byte offset per lane (at most 8 rows of K_pad or
+    // T_pad floats: the host checks that a row of either fits 2^28 floats)
+    const float *ag = U + (size_t)f * C_pad * K_pad + (size_t)kb * BM;
+    const float *bg = V + (size_t)f * C_pad * T_pad + (size_t)tb * BN;
+    const uint32_t aOff = 4u * ((uint32_t)arow * (uint32_t)K_pad + acol), bOff = 4u * ((uint32_t)brow * (uint32_t)T_pad + bcol);
     const size_t aStage = (size_t)BK * K_pad, bStage = (size_t)BK * T_pad;
     const int aLds = arow * BM + acol, bLds = brow * BN + bcol;
 
@@ -89,8 +110,8 @@ __device__ __forceinline__ void gemm_tile(const float *__restrict__ U, const flo
 #pragma unroll
     for (int u = 0; u < PF; u++)
         if (u < nStages) {
-            load_rows(ra[u], ag + (size_t)u * aStage, aPass, SeqA());
-            load_rows(rb[u], bg + (size_t)u * bStage, bPass, SeqB());
+            load_rows(ra[u], ag + (size_t)u * aStage, aOff, aPass, SeqA());
+            load_rows(rb[u], bg + (size_t)u * bStage, bOff, bPass, SeqB());
         }
 
     floatx16 acc[MI][NI];
@@ -104,9 +125,11 @@ __device__ __forceinline__ void gemm_tile(const float *__restrict__ U, const flo
     store_rows(As0 + aLds, ra[0], TL::A_ROWS * BM, SeqA());
     store_rows(Bs0 + bLds, rb[0], TL::B_ROWS * BN, SeqB());
     if (PF < nStages) {
-        load_rows(ra[0], ag + (size_t)PF * aStage, aPass, SeqA());
-        load_rows(rb[0], bg + (size_t)PF * bStage, bPass, SeqB());
+        load_rows(ra[0], ag + (size_t)PF * aStage, aOff, aPass, SeqA());
+        load_rows(rb[0], bg + (size_t)PF * bStage, bOff, bPass, SeqB());
     }
+    // the stage the loop fetches next: stage 1 + PF, advanced by one stage per fetch
+    const float *agNext = uniform_ptr(ag + (size_t)(1 + PF) * aStage), *bgNext = uniform_ptr(bg + (size_t)(1 + PF) * bStage);
     __syncthreads();
 
     // fragment addresses: lane l reads element (row kk + l/32, column base + l%32)
@@ -120,39 +143,72 @@ __device__ __forceinline__ void gemm_tile(const float *__restrict__ U, const flo
         const float *as = As0 + buf * (BK * BM), *bs = Bs0 + buf * (BK * BN);
         const bool more = s + 1 < nStages;
         constexpr int un = (u + 1) % PF;
-        // the fragments of step kk+2 are fetched from LDS before the MFMAs of step kk are issued
-        float a[2][MI], bb[2][NI];
+        // Fragments are fetched two reduction steps (kk, kk+2) at a time, a pair ahead of the MFMAs that use them.
+        // The two reads of a pair are 2*BM (2*BN) floats apart, a multiple of 64 dwords: one ds_read2st64 with both
+        // offsets as immediates off the stage's base register, where a pair of neighbouring 32-wide blocks needed
+        // a vector add per step for its address.
+        // (one base register per 32-wide block, made opaque: seen as base + 32 dwords the compiler pairs
+        // neighbouring blocks again)
+        typedef const __attribute__((address_space(3))) float *LdsPtr;
+        LdsPtr asb[MI], bsb[NI];
 #pragma unroll
-        for (int mi = 0; mi < MI; mi++) a[0][mi] = as[aFrag + mi * 32];
+        for (int mi = 0; mi < MI; mi++) {
+            asb[mi] = (LdsPtr)(as + aFrag + mi * 32);
+            asm volatile("" : "+v"(asb[mi]));
+        }
 #pragma unroll
-        for (int ni = 0; ni < NI; ni++) bb[0][ni] = bs[bFrag + ni * 32];
+        for (int ni = 0; ni < NI; ni++) {
+            bsb[ni] = (LdsPtr)(bs + bFrag + ni * 32);
+            asm volatile("" : "+v"(bsb[ni]));
+        }
+        float a[2][2][MI], bb[2][2][NI];
 #pragma unroll
-        for (int kk = 0; kk < BK; kk += 2) {
-            const int cur = (kk >> 1) & 1, nxt = cur ^ 1;
-            if (kk + 2 < BK) {
+        for (int mi = 0; mi < MI; mi++) {
+            a[0][0][mi] = asb[mi][0];
+            a[0][1][mi] = asb[mi][2 * BM];
+        }
 #pragma unroll
-                for (int mi = 0; mi < MI; mi++) a[nxt][mi] = as[aFrag + (kk + 2) * BM + mi * 32];
+        for (int ni = 0; ni < NI; ni++) {
+            bb[0][0][ni] = bsb[ni][0];
+            bb[0][1][ni] = bsb[ni][2 * BN];
+        }
 #pragma unroll
-                for (int ni = 0; ni < NI; ni++) bb[nxt][ni] = bs[bFrag + (kk + 2) * BN + ni * 32];
+        for (int kq = 0; kq < BK / 4; kq++) {
+            const int cur = kq & 1, nxt = cur ^ 1;
+            if (kq + 1 < BK / 4) {
+#pragma unroll
+                for (int mi = 0; mi < MI; mi++) {
+                    a[nxt][0][mi] = asb[mi][(4 * kq + 4) * BM];
+                    a[nxt][1][mi] = asb[mi][(4 * kq + 6) * BM];
+                }
+#pragma unroll
+                for (int ni = 0; ni < NI; ni++) {
+                    bb[nxt][0][ni] = bsb[ni][(4 * kq + 4) * BN];
+                    bb[nxt][1][ni] = bsb[ni][(4 * kq + 6) * BN];
+                }
             }
 #pragma unroll
-            for (int mi = 0; mi < MI; mi++)
+            for (int st = 0; st < 2; st++)
 #pragma unroll
-                for (int ni = 0; ni < NI; ni++)
-                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][mi], bb[cur][ni], acc[mi][ni], 0, 0, 0);
-            if (kk + 2 < BK) {
+                for (int mi = 0; mi < MI; mi++)
+#pragma unroll
+                    for (int ni = 0; ni < NI; ni++)
+                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][st][mi], bb[cur][st][ni], acc[mi][ni], 0, 0, 0);
+            if (kq + 1 < BK / 4) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                 __builtin_amdgcn_sched_group_barrier(0x100, MI + NI, 0);
-                __builtin_amdgcn_sched_group_barrier(0x008, MI * NI - 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 2 * MI * NI - 1, 0);
             }
-            if (kk == BK / 2 && more) {
+            if (4 * kq == BK / 2 && more) {
                 // the next stage goes to the other LDS buffer half way through this one's MFMAs,
                 // and its registers are refilled with the stage PF further on
                 store_rows(As0 + (buf ^ 1) * (BK * BM) + aLds, ra[un], TL::A_ROWS * BM, SeqA());
                 store_rows(Bs0 + (buf ^ 1) * (BK * BN) + bLds, rb[un], TL::B_ROWS * BN, SeqB());
                 if (s + 1 + PF < nStages) {
-                    load_rows(ra[un], ag + (size_t)(s + 1 + PF) * aStage, aPass, SeqA());
-                    load_rows(rb[un], bg + (size_t)(s + 1 + PF) * bStage, bPass, SeqB());
+                    load_rows(ra[un], agNext, aOff, aPass, SeqA());
+                    load_rows(rb[un], bgNext, bOff, bPass, SeqB());
+                    agNext = uniform_ptr(agNext + aStage);
+                    bgNext = uniform_ptr(bgNext + bStage);
                 }
             }
         }
@@ -164,16 +220,22 @@ __device__ __forceinline__ void gemm_tile(const float *__restrict__ U, const flo
     stage_rest(stage, s0, nStages, std::make_integer_sequence<int, PF - 1>());
 
     // D block layout: register i of lane l is row 8*(i/4) + 4*(l/32) + i%4, column l%32.
-    float *Mg = M + ((size_t)f * K_pad + (size_t)kb * BM + wm0) * T_pad + (size_t)tb * BN + wn0;
+    // The wavefront's block starts at a uniform address; the lane's share of it (4 * lrow rows down, lcol columns in) is one byte offset.
+    float *Mg = (M + ((size_t)f * K_pad + (size_t)kb * BM + wm0) * T_pad + (size_t)tb * BN + wn0);
+    const uint32_t mOff = 4u * (4u * (uint32_t)lrow * (uint32_t)T_pad + lcol);
+    const size_t rowBytes = (size_t)T_pad * 4;
 #pragma unroll
     for (int mi = 0; mi < MI; mi++)
 #pragma unroll
-        for (int ni = 0; ni < NI; ni++)
+        for (int ni = 0; ni < NI; ni++) {
+            // rows 0-3, 8-11, 16-19, 24-27 of the 32x32 block, stepped by addition in the scalar unit
+            char *pr = reinterpret_cast<char *>(uniform_ptr(Mg + (size_t)(mi * 32) * T_pad + ni * 32));
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                const int row = mi * 32 + 8 * (i / 4) + 4 * lrow + (i % 4);
-                Mg[(size_t)row * T_pad + ni * 32 + lcol] = acc[mi][ni][i];
+                *reinterpret_cast<float *>(pr + mOff) = acc[mi][ni][i];
+                pr = uniform_ptr(pr + ((i % 4) == 3 ? 5 * rowBytes : rowBytes));
             }
+        }
 }
 
 // Workgroups are dealt to the 8 XCDs round-robin by linear id.  All tiles of one
