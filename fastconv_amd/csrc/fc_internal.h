@@ -142,3 +142,16 @@ __device__ __forceinline__ uint32_t fc_div(uint32_t n, const fc_fastdiv f) {
     const uint32_t t = __umulhi(n, f.mul);
     return (t + ((n - t) >> 1)) >> (f.shift - 1);
 }
+
+// A pointer that is the same for every lane, pinned to scalar registers: without the pin the
+// compiler turns a uniform base that advances in a loop into a 64-bit pointer per lane and pays
+// a vector add per access.
+template <class T>
+__device__ __forceinline__ T *uniform_ptr(T *p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    // through a global-memory pointer type: rebuilt from an integer the pointer would otherwise be a generic one
+    typedef __attribute__((address_space(1))) T GlobalT;
+    return (T *)reinterpret_cast<GlobalT *>(((uint64_t)hi << 32) | lo);
+}
+

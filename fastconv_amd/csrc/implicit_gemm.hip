@@ -100,6 +100,15 @@ __device__ __forceinline__ void ig_load_rows(floatx4 (&r)[sizeof...(I)], const f
                                              std::integer_sequence<int, I...>) {
     ((r[I] = *reinterpret_cast<const floatx4 *>(p + (size_t)I * rowStride)), ...);
 }
+// The same from a base all lanes share (scalar registers) and one 32-bit byte offset per lane: no vector
+// instruction goes into the addresses (see load_rows in wino_gemm.hip).
+template <int... I>
+__device__ __forceinline__ void ig_load_rows_at(floatx4 (&r)[sizeof...(I)], const float *base, uint32_t laneOff, size_t rowStride,
+                                                std::integer_sequence<int, I...>) {
+    asm volatile("" : "+v"(laneOff));
+    const float *b = uniform_ptr(base);
+    ((r[I] = *reinterpret_cast<const floatx4 *>(reinterpret_cast<const char *>(b) + laneOff), b = uniform_ptr(b + rowStride)), ...);
+}
 template <int... I>
 __device__ __forceinline__ void ig_store_rows(float *lds, const floatx4 (&r)[sizeof...(I)], int rowStride,
                                               std::integer_sequence<int, I...>) {
@@ -196,7 +205,8 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
 
     // filter tile: straight 16-byte copies
     const int arow = tid / (BM / 4), acol = (tid % (BM / 4)) * 4;
-    const float *ag = p.Wp + (size_t)arow * p.K_pad + (size_t)kb * BM + acol;
+    const float *ag = p.Wp + (size_t)kb * BM;                     // uniform; the lane adds aOff bytes
+    const uint32_t aOff = 4u * ((uint32_t)arow * (uint32_t)p.K_pad + acol);
     const size_t aStage = (size_t)BK * p.K_pad, aPass = (size_t)TL::A_ROWS * p.K_pad;
     const int aLds = arow * BM + acol;
 
@@ -243,11 +253,12 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
     using SeqBV = std::make_integer_sequence<int, BV_LD>;
     const int vrow = tid / (BN / 4), vcol = (tid % (BN / 4)) * 4;
     const int HW = p.H * p.W;
-    const float *vg = p.x;
+    const float *vg = p.x;      // uniform; the lane adds vOff bytes (the pointwise path is taken for inputs below 4 GiB)
+    uint32_t vOff = 0;
     if (PW) {
         const long pix4 = min((long)pb * BN + vcol, p.Npix - 4);
         const uint32_t n = fc_div((uint32_t)pix4, p.divOHW);
-        vg = p.x + ((size_t)n * p.C + vrow) * HW + ((uint32_t)pix4 - n * (uint32_t)HW);
+        vOff = 4u * ((n * (uint32_t)p.C + vrow) * (uint32_t)HW + ((uint32_t)pix4 - n * (uint32_t)HW));
     }
     const size_t vPass = (size_t)BV_ROWS * HW, vStage = (size_t)BK * HW;
     const int vLds = vrow * BN + vcol;
@@ -295,10 +306,10 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
         }
     };
     ag += (size_t)sBegin * aStage;
-    ig_load_rows(ra, ag, aPass, SeqA());
+    ig_load_rows_at(ra, ag, aOff, aPass, SeqA());
     if (PW) {
         vg += (size_t)sBegin * vStage;
-        ig_load_rows(rv, vg, vPass, SeqBV());
+        ig_load_rows_at(rv, vg, vOff, vPass, SeqBV());
     } else if (TAP) {
         tap_gather();
     } else if (BUF) {
@@ -318,10 +329,16 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
     ig_store_rows(&As[0][aLds], ra, TL::A_ROWS * BM, SeqA());
     if (PW) ig_store_rows(&Bs[0][vLds], rv, BV_ROWS * BN, SeqBV());
     else ig_scatter_rows<!BUF>(&Bs[0][bLds], rb, rbOk, TL::ROW_STEP * BN, SeqB());
-    // stage s of the reduction into the staging registers
+    // stage s of the reduction into the staging registers (stages are requested in order: the operands' bases are
+    // running pointers in scalar registers, one stage further per call)
+    const float *agNext = uniform_ptr(ag + aStage), *vgNext = uniform_ptr(vg + vStage);
     auto load_stage = [&](const int s) __attribute__((always_inline)) {
-        ig_load_rows(ra, ag + (size_t)(s - sBegin) * aStage, aPass, SeqA());
-        if (PW) ig_load_rows(rv, vg + (size_t)(s - sBegin) * vStage, vPass, SeqBV());
+        ig_load_rows_at(ra, agNext, aOff, aPass, SeqA());
+        agNext = uniform_ptr(agNext + aStage);
+        if (PW) {
+            ig_load_rows_at(rv, vgNext, vOff, vPass, SeqBV());
+            vgNext = uniform_ptr(vgNext + vStage);
+        }
         else if (TAP) tap_gather();
         else if (BUF) ig_gather_rows_buf<true>(rb, xres, pixByte, invLo, invHi, p.table, s * BK + grow0, TL::ROW_STEP, p.kw, SeqB());
         else rbOk = ig_gather_rows<true>(rb, ximg, pixOff, maskR, maskS, p.table, s * BK + grow0, TL::ROW_STEP, SeqB());
@@ -335,33 +352,56 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
         const int buf = (s - sBegin) & 1;
         const float *as = As[buf], *bs = Bs[buf];
         const bool more = s + 1 < sEnd;
-        float a[2][MI], bb[2][NI];
+        // fragments two reduction steps (kk, kk+2) at a time, a pair ahead of their MFMAs: one ds_read2st64 per
+        // 32-wide block and pair, both offsets immediates off an opaque base register (see wino_gemm.hip)
+        typedef const __attribute__((address_space(3))) float *LdsPtr;
+        LdsPtr asb[MI], bsb[NI];
 #pragma unroll
-        for (int mi = 0; mi < MI; mi++) a[0][mi] = as[aFrag + mi * 32];
+        for (int mi = 0; mi < MI; mi++) {
+            asb[mi] = (LdsPtr)(as + aFrag + mi * 32);
+            asm volatile("" : "+v"(asb[mi]));
+        }
 #pragma unroll
-        for (int ni = 0; ni < NI; ni++) bb[0][ni] = bs[bFrag + ni * 32];
+        for (int ni = 0; ni < NI; ni++) {
+            bsb[ni] = (LdsPtr)(bs + bFrag + ni * 32);
+            asm volatile("" : "+v"(bsb[ni]));
+        }
+        float a[2][2][MI], bb[2][2][NI];
 #pragma unroll
-        for (int kk = 0; kk < BK; kk += 2) {
-            const int cur = (kk >> 1) & 1, nxt = cur ^ 1;
-            if (kk + 2 < BK) {
+        for (int mi = 0; mi < MI; mi++) {
+            a[0][0][mi] = asb[mi][0];
+            a[0][1][mi] = asb[mi][2 * BM];
+        }
 #pragma unroll
-                for (int mi = 0; mi < MI; mi++) a[nxt][mi] = as[aFrag + (kk + 2) * BM + mi * 32];
+        for (int ni = 0; ni < NI; ni++) {
+            bb[0][0][ni] = bsb[ni][0];
+            bb[0][1][ni] = bsb[ni][2 * BN];
+        }
 #pragma unroll
-                for (int ni = 0; ni < NI; ni++) bb[nxt][ni] = bs[bFrag + (kk + 2) * BN + ni * 32];
+        for (int kq = 0; kq < BK / 4; kq++) {
+            const int cur = kq & 1, nxt = cur ^ 1;
+            if (kq + 1 < BK / 4) {
+#pragma unroll
+                for (int mi = 0; mi < MI; mi++) {
+                    a[nxt][0][mi] = asb[mi][(4 * kq + 4) * BM];
+                    a[nxt][1][mi] = asb[mi][(4 * kq + 6) * BM];
+                }
+#pragma unroll
+                for (int ni = 0; ni < NI; ni++) {
+                    bb[nxt][0][ni] = bsb[ni][(4 * kq + 4) * BN];
+                    bb[nxt][1][ni] = bsb[ni][(4 * kq + 6) * BN];
+                }
             }
+            // the reads of the next pair are issued before the MFMAs of this one
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int mi = 0; mi < MI; mi++)
+            for (int st = 0; st < 2; st++)
 #pragma unroll
-                for (int ni = 0; ni < NI; ni++)
-                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][mi], bb[cur][ni], acc[mi][ni], 0, 0, 0);
-            if (kk + 2 < BK) {
-                // after the first MFMA of a step, the LDS reads of the next step: their latency
-                // passes under the remaining MFMAs
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, MI + NI, 0);
-                __builtin_amdgcn_sched_group_barrier(0x008, MI * NI - 1, 0);
-            }
-            if (kk == BK / 2 && more) {
+                for (int mi = 0; mi < MI; mi++)
+#pragma unroll
+                    for (int ni = 0; ni < NI; ni++)
+                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][st][mi], bb[cur][st][ni], acc[mi][ni], 0, 0, 0);
+            if (4 * kq == BK / 2 && more) {
                 // the next stage goes to the other LDS buffer half way through this one's MFMAs,
                 // and the one after it is requested at once: a whole stage in flight
                 ig_store_rows(&As[buf ^ 1][aLds], ra, TL::A_ROWS * BM, SeqA());
@@ -502,7 +542,7 @@ void launch(fc_context *ctx, IgemmParams &p) {
     const dim3 grid((unsigned)(((p.nKB * p.nPB + 7) / 8) * 8), (unsigned)p.splitK);
     const bool pointwise = p.kh == 1 && p.kw == 1 && p.sh == 1 && p.sw == 1 && p.pt == 0 && p.pl == 0 &&
                            p.OH == p.H && p.OW == p.W && (p.H * p.W) % 4 == 0 && p.C % TL::BK_ == 0 &&
-                           ((uintptr_t)p.x & 15) == 0;
+                           ((uintptr_t)p.x & 15) == 0 && p.xBytes < (1l << 32);
     // no tap of any window leaves the image, and no padding rows in the reduction
     const bool inside = p.pt == 0 && p.pl == 0 && (p.OH - 1) * p.sh + p.kh <= p.H && (p.OW - 1) * p.sw + p.kw <= p.W &&
                         (p.C * p.kh * p.kw) % TL::BK_ == 0;

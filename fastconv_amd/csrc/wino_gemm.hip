@@ -19,18 +19,6 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 // and the tile makes a round trip through scratch memory.
 // `base` is the same for the whole workgroup (it stays in scalar registers); a lane adds its
 // 32-bit byte offset: no vector instruction goes into the addresses.
-// A pointer that is the same for every lane, pinned to scalar registers: without the pin the
-// compiler turns a uniform base that advances in a loop into a 64-bit pointer per lane and pays
-// a vector add per access.
-template <class T>
-__device__ __forceinline__ T *uniform_ptr(T *p) {
-    const uint64_t v = reinterpret_cast<uint64_t>(p);
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    // through a global-memory pointer type: rebuilt from an integer the pointer would otherwise be a generic one
-    typedef __attribute__((address_space(1))) T GlobalT;
-    return (T *)reinterpret_cast<GlobalT *>(((uint64_t)hi << 32) | lo);
-}
-
 template <int... I>
 __device__ __forceinline__ void load_rows(floatx4 (&r)[sizeof...(I)], const float *base, uint32_t laneOff, size_t rowStride,
                                           std::integer_sequence<int, I...>) {
@@ -187,6 +175,8 @@ __device__ __forceinline__ void gemm_tile(const float *__restrict__ U, const flo
                     bb[nxt][1][ni] = bsb[ni][(4 * kq + 6) * BN];
                 }
             }
+            // the reads of the next pair are issued before the MFMAs of this one (the scheduler would put them behind)
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int st = 0; st < 2; st++)
 #pragma unroll
@@ -194,11 +184,6 @@ __device__ __forceinline__ void gemm_tile(const float *__restrict__ U, const flo
 #pragma unroll
                     for (int ni = 0; ni < NI; ni++)
                         acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][st][mi], bb[cur][st][ni], acc[mi][ni], 0, 0, 0);
-            if (kq + 1 < BK / 4) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, MI + NI, 0);
-                __builtin_amdgcn_sched_group_barrier(0x008, 2 * MI * NI - 1, 0);
-            }
             if (4 * kq == BK / 2 && more) {
                 // the next stage goes to the other LDS buffer half way through this one's MFMAs,
                 // and its registers are refilled with the stage PF further on
