@@ -75,6 +75,7 @@ WORKLOADS = {
     "conv64_224_b32": (_w([(64, 64, 224, 1)]), 32, "winograd", "single 3x3 conv 64->64 @224, batch 32 (VGG-16 layer 2)"),
     "conv256_56_b32": (_w([(256, 256, 56, 1)]), 32, "winograd", "single 3x3 conv 256->256 @56, batch 32 (VGG-16 layers 6-7)"),
     "conv512_28_b32": (_w([(512, 512, 28, 1)]), 32, "winograd", "single 3x3 conv 512->512 @28, batch 32 (VGG-16 layers 9-10)"),
+    "conv512_14_b1": (_w([(512, 512, 14, 1)]), 1, "winograd", "single 3x3 conv 512->512 @14, batch 1 (VGG-16 layers 11-13): 9 tiles"),
     "igemm_3x3s2_b32": ([(128, 128, 56, 3, 2, 1, 1)], 32, "im2col", "single 3x3 stride-2 conv 128->128 @56, implicit GEMM, batch 32 (ResNet-50 conv3 entry)"),
     "igemm_1x1_b32": ([(256, 64, 56, 1, 1, 0, 1)], 32, "im2col", "single 1x1 conv 256->64 @56, implicit GEMM, batch 32 (ResNet-50 bottleneck reduce)"),
     "igemm_stem_b32": ([(3, 64, 224, 7, 2, 3, 1)], 32, "im2col", "single 7x7 stride-2 conv 3->64 @224, implicit GEMM, batch 32 (ResNet-50 stem)"),
@@ -184,6 +185,13 @@ def forward(L, lay, V, M, filter_ready=False):
                                      filter_ready=filter_ready or n0 > 0)
     else:
         L.wino_forward(lay.plan, lay.x, lay.w, lay.U, V, M, lay.y, filter_ready=filter_ready)
+
+
+def takes_raw_filter_gemm(L, lay, filter_ready):
+    """The staged pipeline multiplies straight from the 3x3 filter (no filter transform, no U) when the layer
+    has few tiles and the filter is not transformed beforehand: the rule fc_wino_forward applies."""
+    return (lay.algo == "winograd" and lay.pipe == "staged" and not lay.fused and not filter_ready
+            and lay.block_plans is None and L.wino_prefer_raw_filter_gemm(lay.plan))
 
 
 def _time(L, fn, iters):
@@ -508,7 +516,11 @@ def run_workload(name, steps, warmup, o, detail=True, offline_filter=None):
             roofline.update(peak_at_measured_clock=round(at_clock, 1), frac_at_measured_clock=round(ach / at_clock, 4))
     transforms = {}
     # online filter transforms of the staged and fused pipelines ride in the input transform's launch
-    merged = [l for l in wino if l.pipe != "onepass"] if not filter_ready else []
+    raw = [l for l in staged if takes_raw_filter_gemm(L, l, filter_ready)]
+    if raw:
+        roofline["kernel"] = "wino_gemm_kernel, wino_rawfilter_gemm_kernel (%d of %d launches per step)" % (
+            sum(l.repeats for l in raw), launches_step)
+    merged = [l for l in wino if l.pipe != "onepass" and l not in raw] if not filter_ready else []
     for tname, idx, key in (("input_transform", ST_IT, "it_bytes"), ("output_transform", ST_OT, "ot_bytes"),
                             ("filter_transform", ST_KT, "kt_bytes")):
         ms, cnt = stage[idx]
@@ -518,7 +530,7 @@ def run_workload(name, steps, warmup, o, detail=True, offline_filter=None):
             elif idx == ST_IT:
                 who = [l for l in wino if l.pipe != "onepass"]
             else:
-                who = [l for l in wino if l not in merged]
+                who = [l for l in wino if l not in merged and l not in raw]
             per_step = max(1, sum(l.repeats * (1 if idx != ST_IT or l.block_plans is None
                                                else -(-l.N // l.img_block)) for l in who))
             b = sum(l.algorithmic()[key] * l.repeats for l in who)
@@ -675,12 +687,15 @@ def run_workload(name, steps, warmup, o, detail=True, offline_filter=None):
                 st[ST_IT] = st[ST_OT] = 0.0
             total = sum(st)
             a = lay.algorithmic()
+            raw_gemm = takes_raw_filter_gemm(L, lay, filter_ready)
+            if raw_gemm:
+                row["gemm_kernel"] = "wino_rawfilter_gemm_kernel (U formed in registers from the 3x3 filter)"
             row.update({
                 "pipeline": lay.pipe, "ms": round(total, 4),
                 "gflops": round(lay.flops / (total * 1e-3) / 1e9, 1),
                 "gemm_tflops": round(a["gemm_flops"] / (st[ST_GEMM] * 1e-3) / 1e12, 2),
                 "gemm_frac_mfma": round(a["gemm_flops"] / (st[ST_GEMM] * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 3),
-                "input_tran_gbs": round((a["it_bytes"] + (0 if st[ST_KT] else a["kt_bytes"])) / (st[ST_IT] * 1e-3) / 1e9, 0)
+                "input_tran_gbs": round((a["it_bytes"] + (0 if st[ST_KT] or raw_gemm else a["kt_bytes"])) / (st[ST_IT] * 1e-3) / 1e9, 0)
                 if st[ST_IT] else None,
                 "output_tran_gbs": round(a["ot_bytes"] / (st[ST_OT] * 1e-3) / 1e9, 0) if st[ST_OT] else None,
                 "stage_ms": {"kernel_tran": round(st[ST_KT], 4), "input_tran": round(st[ST_IT], 4),

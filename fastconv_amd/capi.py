@@ -97,6 +97,9 @@ _ABI = {
     "fc_wino_filter_transform": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp]),
     "fc_wino_input_transform": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp]),
     "fc_wino_gemm": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, _vp]),
+    "fc_wino_gemm_raw_filter": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, _vp, C.c_int, C.c_int]),
+    "fc_wino_raw_filter_gemm_applies": (C.c_int, [C.POINTER(WinoPlan)]),
+    "fc_wino_prefer_raw_filter_gemm": (C.c_int, [C.POINTER(WinoPlan)]),
     "fc_wino_output_transform": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, C.c_int, _vp]),
     "fc_wino_filter_input_transform": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, _vp, _vp]),
     "fc_wino_gemm_output_fused": (C.c_int, [_vp, C.POINTER(WinoPlan), _vp, _vp, _vp, C.c_int, _vp]),
@@ -353,6 +356,15 @@ class Library:
 
     def wino_gemm(self, plan, U, V, M):
         self._check(self.c.fc_wino_gemm(self.ctx, C.byref(plan), U, V, M))
+
+    def wino_gemm_raw_filter(self, plan, w, V, M, freqs_per_wave=0, channel_split=0):
+        self._check(self.c.fc_wino_gemm_raw_filter(self.ctx, C.byref(plan), w, V, M, int(freqs_per_wave), int(channel_split)))
+
+    def wino_raw_filter_gemm_applies(self, plan):
+        return bool(self.c.fc_wino_raw_filter_gemm_applies(C.byref(plan)))
+
+    def wino_prefer_raw_filter_gemm(self, plan):
+        return bool(self.c.fc_wino_prefer_raw_filter_gemm(C.byref(plan)))
 
     def wino_output_transform(self, plan, M, y, bias=None, relu=False):
         self._check(self.c.fc_wino_output_transform(self.ctx, C.byref(plan), M, bias, int(relu), y))

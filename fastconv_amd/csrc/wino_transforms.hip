@@ -405,10 +405,11 @@ extern "C" int fc_wino_make_plan(const fc_conv_shape *s, int gemm_config, fc_win
 
 // Measured on MI355X (both algorithms at their best tile shape, whole-layer forward time, every 3x3
 // stride-1 layer of VGG-16 and ResNet-50 at batch 1 and 32): Winograd wins on every layer with at
-// least 1.85 GFLOP of direct-convolution work and 16 or more input channels (by 1.25x to 3.9x), the
-// implicit GEMM on every layer of 0.92 GFLOP or less (batch-1 layers: one launch against three, and no
-// 64x larger transformed filter to write and read); on the 3-channel first layer the two are level at
-// batch 32 (both bound by the stores of the output) and the implicit GEMM is 2.1x ahead at batch 1.
+// least 1.85 GFLOP of direct-convolution work and 16 or more input channels (by 1.25x to 3.9x); on the
+// batch-1 layers of 0.92 GFLOP or less one implicit-GEMM launch is level with the three launches of
+// the staged pipeline (within 4 % on three of five layers, 1.2-1.4x ahead on two) and is what the rule
+// takes; on the 3-channel first layer the two are level at batch 32 (both bound by the stores of the
+// output) and the implicit GEMM is 2.1x ahead at batch 1.
 extern "C" int fc_prefer_winograd(const fc_conv_shape *s) {
     if (!fc_shape_ok(s) || s->kh != 3 || s->kw != 3 || s->sh != 1 || s->sw != 1) return 0;
     const int OH = fc_out_dim(s->H, s->pt, s->pb, 3, 1), OW = fc_out_dim(s->W, s->pl, s->pr, 3, 1);
@@ -562,8 +563,17 @@ extern "C" int fc_wino_output_transform(fc_context *ctx, const fc_wino_plan *pla
 extern "C" int fc_wino_forward(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev, const float *w_dev,
                                const float *bias_dev, int relu, int filter_ready, float *U_dev, float *V_dev,
                                float *M_dev, float *y_dev) {
-    int rc = filter_ready ? fc_wino_input_transform(ctx, plan, x_dev, V_dev)
-                          : fc_wino_filter_input_transform(ctx, plan, w_dev, U_dev, x_dev, V_dev);
+    int rc;
+    if (!filter_ready && w_dev && fc_wino_prefer_raw_filter_gemm(plan)) {
+        // few tiles and no transformed filter yet: the products are made from the 9 filter taps, U is not written
+        rc = fc_wino_input_transform(ctx, plan, x_dev, V_dev);
+        if (rc) return rc;
+        rc = fc_wino_gemm_raw_filter(ctx, plan, w_dev, V_dev, M_dev, 0, 0);
+        if (rc) return rc;
+        return fc_wino_output_transform(ctx, plan, M_dev, bias_dev, relu, y_dev);
+    }
+    rc = filter_ready ? fc_wino_input_transform(ctx, plan, x_dev, V_dev)
+                      : fc_wino_filter_input_transform(ctx, plan, w_dev, U_dev, x_dev, V_dev);
     if (rc) return rc;
     rc = fc_wino_gemm(ctx, plan, U_dev, V_dev, M_dev);
     if (rc) return rc;

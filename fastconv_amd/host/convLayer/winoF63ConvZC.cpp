@@ -84,9 +84,13 @@ void ConvWinoF63ZCLayer::RunOnce(bool filter_ready) {
 // per-stage times, which the reference prints one by one.
 void ConvWinoF63ZCLayer::RunStages(bool filter_ready) {
     Device &d = Device::Get();
-    if (!filter_ready) d.Check(fc_wino_filter_transform(d.ctx(), &plan, dev.kernel, kernelBuf), "fc_wino_filter_transform");
+    // few tiles and an online filter: the products are made straight from the 3x3 taps (as RunOnce does)
+    const bool raw = !filter_ready && fc_wino_prefer_raw_filter_gemm(&plan);
+    if (!filter_ready && !raw)
+        d.Check(fc_wino_filter_transform(d.ctx(), &plan, dev.kernel, kernelBuf), "fc_wino_filter_transform");
     d.Check(fc_wino_input_transform(d.ctx(), &plan, dev.input, inputBuf), "fc_wino_input_transform");
-    d.Check(fc_wino_gemm(d.ctx(), &plan, kernelBuf, inputBuf, gemmBuf), "fc_wino_gemm");
+    if (raw) d.Check(fc_wino_gemm_raw_filter(d.ctx(), &plan, dev.kernel, inputBuf, gemmBuf, 0, 0), "fc_wino_gemm_raw_filter");
+    else d.Check(fc_wino_gemm(d.ctx(), &plan, kernelBuf, inputBuf, gemmBuf), "fc_wino_gemm");
     d.Check(fc_wino_output_transform(d.ctx(), &plan, gemmBuf, dev.bias, relu ? 1 : 0, dev.output), "fc_wino_output_transform");
 }
 

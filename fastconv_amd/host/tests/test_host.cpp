@@ -113,15 +113,15 @@ static void test_select_algorithm() {
     // layers where the two are within 15 % of each other may go either way (boxes of the pool differ by up to that
     // much on layers bound by their stores, such as the 3-channel first layer)
     static const struct { int c, k, h, n; double wino_ms, im2col_ms; } measured[] = {
-        {3, 64, 224, 1, 0.0254, 0.0117}, {64, 64, 224, 1, 0.0370, 0.0518}, {64, 128, 112, 1, 0.0298, 0.0386},
-        {128, 128, 112, 1, 0.0336, 0.0554}, {128, 256, 56, 1, 0.0299, 0.0375}, {256, 256, 56, 1, 0.0341, 0.0532},
-        {256, 512, 28, 1, 0.0316, 0.0348}, {512, 512, 28, 1, 0.0397, 0.0517}, {512, 512, 14, 1, 0.0402, 0.0314},
-        {64, 64, 56, 1, 0.0194, 0.0165}, {128, 128, 28, 1, 0.0191, 0.0199}, {256, 256, 14, 1, 0.0271, 0.0223},
-        {512, 512, 7, 1, 0.0404, 0.0215}, {3, 64, 224, 32, 0.1187, 0.1306}, {64, 64, 224, 32, 0.4947, 1.0407},
-        {64, 128, 112, 32, 0.2671, 0.4820}, {128, 128, 112, 32, 0.4241, 0.9511}, {128, 256, 56, 32, 0.2036, 0.4838},
-        {256, 256, 56, 32, 0.3221, 0.9553}, {256, 512, 28, 32, 0.1674, 0.5079}, {512, 512, 28, 32, 0.2994, 1.0145},
-        {512, 512, 14, 32, 0.1342, 0.2886}, {64, 64, 56, 32, 0.0549, 0.0798}, {128, 128, 28, 32, 0.0462, 0.0881},
-        {256, 256, 14, 32, 0.0535, 0.0865}, {512, 512, 7, 32, 0.0735, 0.0866}};
+        {3, 64, 224, 1, 0.0256, 0.0119}, {64, 64, 224, 1, 0.0370, 0.0510}, {64, 128, 112, 1, 0.0300, 0.0376},
+        {128, 128, 112, 1, 0.0326, 0.0567}, {128, 256, 56, 1, 0.0305, 0.0383}, {256, 256, 56, 1, 0.0342, 0.0533},
+        {256, 512, 28, 1, 0.0270, 0.0349}, {512, 512, 28, 1, 0.0344, 0.0511}, {512, 512, 14, 1, 0.0302, 0.0311},
+        {64, 64, 56, 1, 0.0196, 0.0168}, {128, 128, 28, 1, 0.0193, 0.0201}, {256, 256, 14, 1, 0.0216, 0.0220},
+        {512, 512, 7, 1, 0.0306, 0.0214}, {3, 64, 224, 32, 0.1222, 0.1308}, {64, 64, 224, 32, 0.4934, 1.0072},
+        {64, 128, 112, 32, 0.2665, 0.4752}, {128, 128, 112, 32, 0.4265, 0.9336}, {128, 256, 56, 32, 0.1987, 0.4774},
+        {256, 256, 56, 32, 0.3187, 0.9552}, {256, 512, 28, 32, 0.1654, 0.4999}, {512, 512, 28, 32, 0.2967, 1.0109},
+        {512, 512, 14, 32, 0.1338, 0.2825}, {64, 64, 56, 32, 0.0546, 0.0779}, {128, 128, 28, 32, 0.0462, 0.0881},
+        {256, 256, 14, 32, 0.0532, 0.0854}, {512, 512, 7, 32, 0.0726, 0.0852}};
     for (size_t i = 0; i < sizeof measured / sizeof measured[0]; i++) {
         const nnp_size o = {(size_t)measured[i].h, (size_t)measured[i].h};
         const bool wino = select_algorithm(k3, s1, o, measured[i].c, measured[i].k, measured[i].n) == nnp_convolution_algorithm_winograd;

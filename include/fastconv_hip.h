@@ -216,6 +216,26 @@ int fc_wino_filter_input_transform(fc_context *ctx, const fc_wino_plan *plan,
 int fc_wino_gemm(fc_context *ctx, const fc_wino_plan *plan,
                  const float *U_dev, const float *V_dev, float *M_dev);
 
+/* The same stage fed by the untransformed filter w[K][C][3][3]: U = G g G^T is formed
+ * in registers, lane by lane in the layout the MFMA takes its first operand in, and never
+ * exists in memory.  For layers with few tiles (batch 1 on 7x7 to 28x28 images), where
+ * the stage above is one pass over U, 64/9 times the size of w.  Like the reference's
+ * online strategy (kernel transform inside Forward, ConvTest.cpp:230-243) without its
+ * kernelBuf.  Needs plan->T <= 64 and C a multiple of 16
+ * (fc_wino_raw_filter_gemm_applies); freqs_per_wave = 0 lets the library choose how many
+ * of the 64 frequencies a wavefront multiplies (1, 2 or 4) and channel_split = 0 over how
+ * many groups of wavefronts a workgroup spreads the input channels (1, 2 or 4): tuning
+ * parameters like the tile shape of fc_wino_gemm.  M is overwritten; its padding (rows from
+ * K rounded up to 16, columns from T rounded up to 16, 32 or 64) is not written. */
+int fc_wino_gemm_raw_filter(fc_context *ctx, const fc_wino_plan *plan,
+                            const float *w_dev, const float *V_dev, float *M_dev,
+                            int freqs_per_wave, int channel_split);
+int fc_wino_raw_filter_gemm_applies(const fc_wino_plan *plan);
+/* 1 when fc_wino_gemm_raw_filter is expected to beat filter transform + fc_wino_gemm
+ * (measured on MI355X: at most 32 tiles and C*K >= 32768).  Against fc_wino_gemm alone,
+ * with the filter transformed beforehand, the two are level. */
+int fc_wino_prefer_raw_filter_gemm(const fc_wino_plan *plan);
+
 /* Y = A^T m A clipped to the image, written NCHW, with an optional per-channel
  * bias (K floats) and optional ReLU.  Replaces the output transform inside
  * winoF63_v1_single (winoF63ZC/winoF63ZC.cpp:869-973). */
@@ -290,7 +310,9 @@ int fc_wino_prefer_onepass(const fc_conv_shape *shape);
 
 /* All stages back to back: what winoF63_v1_single (winoF63ZC/winoF63ZC.h:5-6)
  * does in one call.  filter_ready != 0 skips the filter transform (U already
- * holds it: the "offline" strategy, ConvTest.cpp:230-243). */
+ * holds it: the "offline" strategy, ConvTest.cpp:230-243).  With filter_ready == 0
+ * the contents of U after the call are unspecified: a layer with few tiles
+ * (fc_wino_prefer_raw_filter_gemm) multiplies straight from w and leaves U alone. */
 int fc_wino_forward(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev,
                     const float *w_dev, const float *bias_dev, int relu, int filter_ready,
                     float *U_dev, float *V_dev, float *M_dev, float *y_dev);

@@ -107,6 +107,70 @@ def test_batch1_real_layers_every_path_against_oracle(lib, C, K, H):
         assert O.max_rel_err(lib.winograd_conv_onepass(cs, x, w), truth) <= TOL_WINO
 
 
+RAW_FILTER_SHAPES = [
+    (1, 512, 14, 14, 512),      # 9 tiles: the deep VGG-16 layers at batch 1
+    (1, 256, 28, 28, 512),      # 25 tiles: two blocks of 16
+    (1, 256, 42, 42, 64),       # 49 tiles: four blocks of 16
+    (1, 16, 6, 6, 5),           # one tile, one chunk of channels, 5 of 16 output channels
+    (2, 48, 12, 12, 20),        # three chunks: the loop tail; output channels not a multiple of 16
+    (1, 80, 7, 7, 33),          # five chunks: one pass of the four-deep pipeline plus a tail
+    (1, 64, 14, 14, 48),
+]
+
+
+@pytest.mark.parametrize("shp", RAW_FILTER_SHAPES)
+def test_winograd_gemm_from_the_untransformed_filter(lib, shp):
+    """fc_wino_gemm_raw_filter (U formed in registers from the 3x3 taps) against the oracle's M and,
+    through the output transform, the fp64 direct convolution, for every choice of frequencies per
+    wavefront and channel split the layer admits."""
+    s = O.shape(*shp)
+    cs = cshape(s)
+    x, w = O.make_inputs(s, seed=shp[1] + shp[4])
+    plan = lib.wino_plan(cs, lib.wino_default_config(cs))
+    assert lib.wino_raw_filter_gemm_applies(plan)
+    T, K, C = plan.T, s.K, s.C
+    Mo = O.wino_gemm(O.wino_filter_transform(w), O.wino_input_transform(s, x))
+    truth = O.naive_conv_f64(s, x, w)
+    nt = 1 if T <= 16 else 2 if T <= 32 else 4
+    splits = [sp for sp in (1, 2, 4) if sp <= {1: 4, 2: 2, 4: 1}[nt] and (C // 16) % sp == 0]
+    mark = lib.mark()
+    try:
+        dx, dw = lib.upload(x), lib.upload(w)
+        V, M = lib.alloc(plan.V_bytes), lib.alloc(plan.M_bytes)
+        y = lib.alloc(4 * s.N * K * plan.OH * plan.OW)
+        lib.wino_input_transform(plan, dx, V)
+        for fpw, sp in [(0, 0)] + [(f, sp) for f in (1, 2, 4) for sp in splits]:
+            announce("raw-filter gemm", shp, "freqs/wave", fpw, "split", sp)
+            lib.wino_gemm_raw_filter(plan, dw, V, M, fpw, sp)
+            Mh = lib.download(M, (64, plan.K_pad, plan.T_pad))
+            assert np.abs(Mh[:, :K, :T] - Mo).max() <= 1e-5 * np.abs(Mo).max()
+            lib.wino_output_transform(plan, M, y)
+            assert O.max_rel_err(lib.download(y, (s.N, K, plan.OH, plan.OW)), truth) <= TOL_WINO
+    finally:
+        lib.release(mark)
+    # the whole-layer call takes this path by itself when it expects it to win
+    assert O.max_rel_err(lib.winograd_conv(cs, x, w), truth) <= TOL_WINO
+
+
+def test_winograd_gemm_from_the_untransformed_filter_refuses_other_layers(lib):
+    import fastconv_amd as F
+    for shp in [(1, 24, 14, 14, 32), (4, 64, 56, 56, 64)]:       # channels not a multiple of 16; 400 tiles
+        cs = cshape(O.shape(*shp))
+        plan = lib.wino_plan(cs, lib.wino_default_config(cs))
+        assert not lib.wino_raw_filter_gemm_applies(plan) and not lib.wino_prefer_raw_filter_gemm(plan)
+        buf = lib.alloc(1 << 20)
+        with pytest.raises(F.FastConvError) as e:
+            lib.wino_gemm_raw_filter(plan, buf, buf, buf)
+        assert e.value.status == -6
+    cs = cshape(O.shape(1, 512, 14, 14, 512))
+    plan = lib.wino_plan(cs, lib.wino_default_config(cs))
+    assert lib.wino_prefer_raw_filter_gemm(plan)
+    buf = lib.alloc(plan.M_bytes)
+    for fpw, sp in [(3, 0), (0, 3), (0, 8)]:
+        with pytest.raises(F.FastConvError):
+            lib.wino_gemm_raw_filter(plan, buf, buf, buf, fpw, sp)
+
+
 def test_winograd_wide_images(lib):
     """Outputs up to 1020 columns (170 tiles per band) are inside the stated limit of the staged
     pipeline; 512 and 1020 columns take the narrower blocks of the input transform."""
