@@ -38,6 +38,18 @@ def test_conv_test_driver_passes_its_own_check(algo):
     assert "PASS" in out and "FAIL" not in out
 
 
+@pytest.mark.parametrize("ts", ["online", "offline"])
+@pytest.mark.parametrize("C,H", [(512, 14), (256, 28)])
+def test_batch1_deep_layers_through_the_staged_layer_class(ts, C, H):
+    """Batch 1 with 9 and 25 tiles through ConvWinoF63ZCLayer: with the online filter transform the
+    products are made straight from the 3x3 filter, with the offline one from the transformed filter."""
+    out = _run([_exe("conv_test"), "-ic", str(C), "-oc", "512", "-is", str(H), str(H), "-ks", "3", "3", "-ip", "1",
+                "-n", "1", "-i", "3", "-t", "16", "-a", "winograd", "-ts", ts, "--strict", "--json"])
+    assert "PASS" in out and "FAIL" not in out
+    j = _json_line(out)
+    assert j["max_rel_err"] <= 1e-3 and j["kernel_transform"] == ts
+
+
 def _json_line(out):
     import json
     return json.loads([l for l in out.splitlines() if l.startswith("{")][-1])
