@@ -83,7 +83,7 @@ WORKLOADS = {
     "stress_b128": (_w(STRESS), 128, "winograd", "VGG-16 256@56, 512@28, 512@14 at batch 128: staged (ZC) against blocked Winograd, tile shapes searched"),
 }
 # (workload, filter transform offline): compact results a default run appends
-SECONDARY = (("vgg16_b1", False), ("vgg16_b1", True), ("resnet50_b32", False), ("im2col_abc_b1", False))
+SECONDARY = (("vgg16_b1", False), ("vgg16_b1", True), ("resnet50_b32", False), ("resnet50_b1", False), ("im2col_abc_b1", False))
 
 ST_KT, ST_IT, ST_GEMM, ST_OT, ST_IGEMM, ST_FUSED, ST_ONEPASS = 0, 1, 2, 3, 4, 6, 7
 
