@@ -30,7 +30,7 @@ struct SmallCParams {
     long T;
     unsigned xBytes; // size of x, at most 2^31
     int tileBlocks, blocksPerXcd;
-    int kPerBlock;   // output channels per workgroup: 64 or 16 (a multiple of 8)
+    int kPerBlock;   // output channels per workgroup: 64, 16 or 8 (a multiple of 8)
     int relu;
     int zero;        // always 0
     fc_fastdiv divTW, divTH;
@@ -346,8 +346,10 @@ int fc_wino_smallc_conv(fc_context *ctx, const fc_wino_plan *plan, const float *
     p.divTH = fc_make_fastdiv(p.tH);
     const int tiles = sc_tiles(s.C);
     const long tileBlocks = (plan->T + tiles - 1) / tiles;
-    // 64 output channels per workgroup when that still gives every CU a few workgroups, else 16
-    p.kPerBlock = tileBlocks * (plan->K_pad / 64) >= 2l * ctx->props.multiProcessorCount ? 64 : 16;
+    // 64 output channels per workgroup when that still gives every CU a few workgroups, else 16, or 8 when even
+    // that leaves CUs without one (batch 1)
+    const long cus = ctx->props.multiProcessorCount;
+    p.kPerBlock = tileBlocks * (plan->K_pad / 64) >= 2 * cus ? 64 : tileBlocks * (plan->K_pad / 16) >= cus ? 16 : 8;
     const long gy = plan->K_pad / p.kPerBlock;
     if (tileBlocks >= (1l << 31) - 8 || gy > 65535)
         return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_conv_onepass: grid too large", hipSuccess);
