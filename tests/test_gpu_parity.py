@@ -152,6 +152,38 @@ def test_winograd_gemm_from_the_untransformed_filter(lib, shp):
     assert O.max_rel_err(lib.winograd_conv(cs, x, w), truth) <= TOL_WINO
 
 
+def test_winograd_gemm_from_the_untransformed_filter_on_random_shapes(lib):
+    """Random small geometries (any padding, output channels and tile counts up to 64, channels a multiple of 16)
+    through input transform, fc_wino_gemm_raw_filter and output transform against the fp64 direct convolution."""
+    rng = np.random.default_rng(7)
+    done = 0
+    while done < 24:
+        N, C, K = int(rng.integers(1, 3)), 16 * int(rng.integers(1, 7)), int(rng.integers(1, 71))
+        H, W, pad = int(rng.integers(3, 25)), int(rng.integers(3, 25)), int(rng.integers(0, 3))
+        if H + 2 * pad < 3 or W + 2 * pad < 3:
+            continue
+        s = O.shape(N, C, H, W, K, 3, 3, 1, 1, pad)
+        cs = cshape(s)
+        plan = lib.wino_plan(cs, lib.wino_default_config(cs))
+        if not lib.wino_raw_filter_gemm_applies(plan):
+            continue
+        done += 1
+        x, w = O.make_inputs(s, seed=100 + done)
+        announce("raw-filter gemm, random shape", (N, C, H, W, K, pad), "tiles", plan.T)
+        mark = lib.mark()
+        try:
+            dx, dw = lib.upload(x), lib.upload(w)
+            V, M = lib.alloc(plan.V_bytes), lib.alloc(plan.M_bytes)
+            y = lib.alloc(4 * N * K * plan.OH * plan.OW)
+            lib.wino_input_transform(plan, dx, V)
+            lib.wino_gemm_raw_filter(plan, dw, V, M)
+            lib.wino_output_transform(plan, M, y)
+            got = lib.download(y, (N, K, plan.OH, plan.OW))
+        finally:
+            lib.release(mark)
+        assert O.max_rel_err(got, O.naive_conv_f64(s, x, w)) <= TOL_WINO
+
+
 def test_winograd_gemm_from_the_untransformed_filter_refuses_other_layers(lib):
     import fastconv_amd as F
     for shp in [(1, 24, 14, 14, 32), (4, 64, 56, 56, 64)]:       # channels not a multiple of 16; 400 tiles
