@@ -665,14 +665,15 @@ extern "C" int fc_igemm_pack_filter(fc_context *ctx, const fc_igemm_plan *plan, 
 
 // Launches of one layer; `timed` brackets the GEMM kernel with events when stage timing is on.
 static int igemm_run(fc_context *ctx, const fc_igemm_plan *plan, const float *x_dev, const float *Wp_dev,
-                     const int32_t *table_dev, const float *bias_dev, int relu, float *ws_dev, float *y_dev, bool timed);
+                     const int32_t *table_dev, const float *bias_dev, int relu, float *ws_dev, float *y_dev, bool timed,
+                     const char *entry);
 
 extern "C" int fc_conv_implicit_gemm(fc_context *ctx, const fc_igemm_plan *plan, const float *x_dev,
                                      const float *Wp_dev, const int32_t *table_dev, const float *bias_dev, int relu,
                                      float *ws_dev, float *y_dev) {
     const int rc = ig_plan_check(ctx, plan);
     if (rc) return rc;
-    return igemm_run(ctx, plan, x_dev, Wp_dev, table_dev, bias_dev, relu, ws_dev, y_dev, true);
+    return igemm_run(ctx, plan, x_dev, Wp_dev, table_dev, bias_dev, relu, ws_dev, y_dev, true, "fc_conv_implicit_gemm");
 }
 
 // ---- the same layer with the split-reduction workspace in a static device array ----
@@ -718,16 +719,21 @@ extern "C" int fc_conv_implicit_gemm_static(fc_context *ctx, const fc_igemm_plan
     if (!ctx->igemm_static_ws) return fc_set_error(ctx, FC_ERR_STATE, "fc_conv_implicit_gemm_static: static workspace not set up", hipSuccess);
     // Nothing has to start at zero: every partial sum the reduction reads ([split][k < K][pixel < Npix]) is
     // written by this call's GEMM kernel first.  No event brackets (creating an event may allocate).
-    return igemm_run(ctx, plan, x_dev, Wp_dev, table_dev, bias_dev, relu, ctx->igemm_static_ws, y_dev, false);
+    return igemm_run(ctx, plan, x_dev, Wp_dev, table_dev, bias_dev, relu, ctx->igemm_static_ws, y_dev, false,
+                     "fc_conv_implicit_gemm_static");
 }
 
 static int igemm_run(fc_context *ctx, const fc_igemm_plan *plan, const float *x_dev, const float *Wp_dev,
-                     const int32_t *table_dev, const float *bias_dev, int relu, float *ws_dev, float *y_dev, bool timed) {
-    if (!x_dev || !Wp_dev || !table_dev || !y_dev)
-        return fc_set_error(ctx, FC_ERR_INVALID, "fc_conv_implicit_gemm: null buffer", hipSuccess);
-    if ((uintptr_t)Wp_dev & 15) return fc_set_error(ctx, FC_ERR_INVALID, "fc_conv_implicit_gemm: Wp must be 16-byte aligned", hipSuccess);
-    if (plan->split_k > 1 && !ws_dev)
-        return fc_set_error(ctx, FC_ERR_INVALID, "fc_conv_implicit_gemm: this plan splits the reduction and needs ws_bytes of workspace", hipSuccess);
+                     const int32_t *table_dev, const float *bias_dev, int relu, float *ws_dev, float *y_dev, bool timed,
+                     const char *entry) {
+    char msg[160];
+    auto fail = [&](int status, const char *what) {
+        snprintf(msg, sizeof msg, "%s: %s", entry, what);
+        return fc_set_error(ctx, status, msg, hipSuccess);
+    };
+    if (!x_dev || !Wp_dev || !table_dev || !y_dev) return fail(FC_ERR_INVALID, "null buffer");
+    if ((uintptr_t)Wp_dev & 15) return fail(FC_ERR_INVALID, "Wp must be 16-byte aligned");
+    if (plan->split_k > 1 && !ws_dev) return fail(FC_ERR_INVALID, "this plan splits the reduction and needs ws_bytes of workspace");
     fc_gemm_config cfg;
     fc_igemm_get_config(plan->config, &cfg);
     const fc_conv_shape &s = plan->shape;
@@ -746,7 +752,7 @@ static int igemm_run(fc_context *ctx, const fc_igemm_plan *plan, const float *x_
     p.ws = ws_dev;
     p.fastStore = s.K % cfg.bm == 0 && 4.0 * s.N * s.K * plan->OH * plan->OW < 4294967296.0 &&
                   4.0 * plan->split_k * s.K * (double)plan->Npix < 4294967296.0 && ((uintptr_t)bias_dev & 15) == 0;
-    if ((long)p.nKB * p.nPB >= (1l << 31)) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_conv_implicit_gemm: grid too large", hipSuccess);
+    if ((long)p.nKB * p.nPB >= (1l << 31)) return fail(FC_ERR_UNSUPPORTED, "grid too large");
     fc_stage_scope scope(ctx, timed ? FC_STAGE_IMPLICIT_GEMM : -1);
     switch (plan->config) {
         case 0: launch<Ig0>(ctx, p); break;
@@ -757,12 +763,12 @@ static int igemm_run(fc_context *ctx, const fc_igemm_plan *plan, const float *x_
         case 5: launch<Ig5>(ctx, p); break;
         case 6: launch<Ig6>(ctx, p); break;
         case 7: launch<Ig7>(ctx, p); break;
-        default: return fc_set_error(ctx, FC_ERR_INVALID, "fc_conv_implicit_gemm: unknown tile configuration", hipSuccess);
+        default: return fail(FC_ERR_INVALID, "unknown tile configuration");
     }
     FC_LAUNCH_CHECK(ctx, "igemm_conv_kernel");
     if (plan->split_k > 1) {
         const dim3 rgrid((unsigned)((plan->Npix + 255) / 256), (unsigned)s.K);
-        if (rgrid.y > 65535) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_conv_implicit_gemm: more than 65535 channels", hipSuccess);
+        if (rgrid.y > 65535) return fail(FC_ERR_UNSUPPORTED, "more than 65535 channels");
         igemm_reduce_kernel<<<rgrid, dim3(256), 0, ctx->stream>>>(ws_dev, bias_dev, y_dev, s.K, plan->Npix,
                                                                   plan->OH * plan->OW, plan->split_k, relu, p.divOHW);
         FC_LAUNCH_CHECK(ctx, "igemm_reduce_kernel");

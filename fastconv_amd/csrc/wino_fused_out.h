@@ -64,6 +64,7 @@ __device__ __forceinline__ void fused_output_transform(const FusedOut &p, const 
             const uint32_t th = fc_div(r, p.divTW), tw = r - th * p.tW;
             const int rows = min(6, p.OH - (int)th * 6), cols = min(6, p.OW - (int)tw * 6);
             const float bias = p.bias ? p.bias[k] : 0.f;
+            // ReLU as a maximum with 0, no ReLU as a maximum with -inf: one v_maximum3_f32 either way, which keeps a NaN
             const float floorv = p.relu ? 0.f : -__builtin_inff();
             float *dst = p.y + (((size_t)n * p.K + k) * p.OH + (size_t)th * 6) * p.OW + tw * 6;
             const bool pairs = cols == 6 && (p.OW & 1) == 0;    // 8-byte aligned row segments
@@ -76,7 +77,7 @@ __device__ __forceinline__ void fused_output_transform(const FusedOut &p, const 
                 at6(rowv, sres);
                 if (i < rows) {
 #pragma unroll
-                    for (int jj = 0; jj < 6; jj++) sres[jj] = fmaxf(sres[jj], floorv);
+                    for (int jj = 0; jj < 6; jj++) sres[jj] = __builtin_elementwise_maximum(sres[jj], floorv);
                     float *drow = dst + (size_t)i * p.OW;
                     if (pairs) {
 #pragma unroll

@@ -176,7 +176,7 @@ __device__ __forceinline__ void sc_step(const SmallCParams &p, const UReg<C> &u,
             float o[6];
             at6(mrow, o);
 #pragma unroll
-            for (int s = 0; s < 6; s++) o[s] = fmaxf(o[s], floorv);
+            for (int s = 0; s < 6; s++) o[s] = __builtin_elementwise_maximum(o[s], floorv);
             if (ROWST) {
                 float2 *sw = reinterpret_cast<float2 *>(st.stage) + lane * 3;
                 wave_sync();   // the previous row has been read by every lane
@@ -272,6 +272,7 @@ __global__ __launch_bounds__(kScThreads) void wino_smallc_kernel(const float *__
     const int kFirst = blockIdx.y * p.kPerBlock + wave * kpw;
     const int kCount = min(kpw, p.K - kFirst);
     if (kCount <= 0) return;
+    // ReLU as a maximum with 0, no ReLU as a maximum with -inf: one v_maximum3_f32 either way, which keeps a NaN
     const float floorv = p.relu ? 0.f : -__builtin_inff();
     ScStore st;
     st.stage = Vs + 64 * TILES * C + wave * kScStageFloats;

@@ -314,6 +314,7 @@ __global__ __launch_bounds__(TPB) void wino_output_transform_kernel(const OutTPa
             for (int i = 0; i < 6; i++) tmp[i][jj] = s[i];
         }
         const float b = p.bias ? p.bias[k] : 0.f;
+        // ReLU as a maximum with 0, no ReLU as a maximum with -inf: one v_maximum3_f32 either way, which keeps a NaN
         const float floorv = p.relu ? 0.f : -__builtin_inff();
         float *img = lds + j * bandElems + q * 6;
         const int colsLeft = p.OW - q * 6;      // columns of this tile inside the image
@@ -324,7 +325,7 @@ __global__ __launch_bounds__(TPB) void wino_output_transform_kernel(const OutTPa
             float s[6];
             at6(row, s);
 #pragma unroll
-            for (int jj = 0; jj < 6; jj++) s[jj] = fmaxf(s[jj], floorv);
+            for (int jj = 0; jj < 6; jj++) s[jj] = __builtin_elementwise_maximum(s[jj], floorv);
             float *dstl = img + i * p.OW;
             if (colsLeft >= 6) {
 #pragma unroll

@@ -110,6 +110,7 @@ Net::Net(size_t arena_bytes) : input_(NULL), graph_(NULL) {
     Device &d = Device::Get();
     arena_mark_ = d.Mark();
     arena_block_ = d.Alloc(arena_bytes, "layer graph arena");
+    arena_top_ = d.Mark();
     alloc_ = new fastconv::RangeAllocator(arena_block_, arena_bytes, 256);
     common_ = new CommonMemPool<float>(alloc_);
 }
@@ -120,10 +121,11 @@ Net::~Net() {
     delete input_;
     delete common_;
     delete alloc_;
-    // the device arena is a stack: the block goes back when nothing was allocated after it
+    // The device arena is a stack: the block goes back only while it is still the top of it.  When
+    // something was allocated after it (and is still alive) the block stays until that owner releases.
     Device &d = Device::Get();
-    size_t cap = 0, used = 0, peak = 0;
-    if (fc_pool_stats(d.pool(), &cap, &used, &peak) == FC_OK && used >= arena_mark_) d.Release(arena_mark_);
+    if (d.Mark() == arena_top_) d.Release(arena_mark_);
+    else fprintf(stderr, "Net: device buffers were allocated after the layer graph arena; its block stays in the pool\n");
 }
 
 void Net::SetInput(size_t n, size_t c, size_t h, size_t w) {

@@ -125,7 +125,8 @@ class Net {
     Blob<float> *input_;
     std::vector<Layer *> layers_;
     void *arena_block_;
-    size_t arena_mark_;
+    size_t arena_mark_;     // pool usage before the arena block was taken
+    size_t arena_top_;      // and right after: the block is the top of the stack while usage equals this
     fc_graph *graph_;
 };
 

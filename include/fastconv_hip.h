@@ -225,8 +225,10 @@ int fc_wino_gemm(fc_context *ctx, const fc_wino_plan *plan,
  * (fc_wino_raw_filter_gemm_applies); freqs_per_wave = 0 lets the library choose how many
  * of the 64 frequencies a wavefront multiplies (1, 2 or 4) and channel_split = 0 over how
  * many groups of wavefronts a workgroup spreads the input channels (1, 2 or 4): tuning
- * parameters like the tile shape of fc_wino_gemm.  M is overwritten; its padding (rows from
- * K rounded up to 16, columns from T rounded up to 16, 32 or 64) is not written. */
+ * parameters like the tile shape of fc_wino_gemm.  M is overwritten: rows K up to K rounded
+ * up to 16 are written as zeros and columns T up to T rounded up to 16, 32 or 64 hold the
+ * products of V's (zero) padding; rows and columns beyond that, up to K_pad and T_pad, are
+ * left as they were.  The output transform reads none of the padding. */
 int fc_wino_gemm_raw_filter(fc_context *ctx, const fc_wino_plan *plan,
                             const float *w_dev, const float *V_dev, float *M_dev,
                             int freqs_per_wave, int channel_split);
@@ -326,8 +328,12 @@ int fc_igemm_get_config(int id, fc_gemm_config *cfg);
 int fc_igemm_default_config(const fc_conv_shape *shape);
 
 /* Filter re-layout done once at Init: Wp[Kred_pad][K_pad], output channel
- * fastest, reduction index (c, r, s) as in the column matrix rows
- * (convLayer/im2colConv.cpp:285-309); plus the per-row gather table. */
+ * fastest, plus the per-row gather table.  The order of the reduction rows is
+ * the library's business and depends on plan->config: the column matrix's
+ * (c, r, s) (convLayer/im2colConv.cpp:285-309) in general, tap-major (r, s, c)
+ * when C is a whole number of the configuration's reduction stages.  Treat Wp
+ * and the table as opaque, hand them only to calls made with the same plan, and
+ * pack them again when the configuration changes. */
 typedef struct {
     fc_conv_shape shape;
     int OH, OW;

@@ -252,6 +252,28 @@ def test_winograd_bias_relu_epilogue(lib):
     assert O.max_rel_err(y, truth) <= TOL_WINO
 
 
+def test_nan_and_inf_reach_the_output_of_every_path(lib):
+    """A NaN in the input must come out as NaN (not as -inf or 0) wherever it contributes, with ReLU
+    off, through the staged, fused, single-kernel and small-channel Winograd epilogues and the
+    implicit GEMM; outputs it does not reach stay finite in the implicit GEMM."""
+    for shp in [(1, 8, 14, 14, 12), (1, 3, 20, 20, 9)]:
+        s = O.shape(*shp)
+        cs = cshape(s)
+        x, w = O.make_inputs(s, seed=3)
+        x[0, 1, 5, 6] = np.nan
+        bias = O.rng_uniform(2, (s.K,))
+        announce("NaN propagation", shp)
+        for name, fn in (("staged", lib.winograd_conv), ("fused", lib.winograd_conv_fused),
+                         ("single kernel", lib.winograd_conv_onepass), ("implicit gemm", lib.implicit_gemm_conv)):
+            y = fn(cs, x, w, bias=bias)
+            assert np.isnan(y[0, :, 4:7, 5:8]).all(), name          # the 3x3 windows that hold the NaN
+            assert not np.isinf(y).any(), name
+            if name == "implicit gemm":
+                ok = np.ones(y.shape, bool)
+                ok[0, :, 4:7, 5:8] = False
+                assert np.isfinite(y[ok]).all()
+
+
 @pytest.mark.parametrize("shp", [
     (2, 3, 8, 11, 5), (1, 64, 56, 56, 64), (3, 10, 14, 14, 70), (2, 16, 7, 7, 33), (1, 8, 30, 20, 40),
     (1, 3, 224, 224, 64), (4, 64, 28, 28, 128), (2, 130, 13, 13, 40),
@@ -325,7 +347,7 @@ def test_winograd_small_channel_kernel(lib, shp, pads):
 
 
 def test_winograd_single_kernel_full_size_layers(lib):
-    for (N, C, H, K) in [(32, 3, 224, 64), (32, 64, 112, 128), (8, 64, 224, 64)]:
+    for (N, C, H, K) in [(32, 3, 224, 64), (32, 64, 112, 128), (8, 64, 224, 64), (32, 64, 224, 64)]:
         s = O.shape(N, C, H, H, K)
         x, w = O.make_inputs(s, seed=2)
         announce("single-kernel full size", (N, C, H, K))
@@ -441,9 +463,15 @@ IGEMM_SHAPES = [
     # ResNet-50 bottleneck layers at batch 32: 1x1 reduce / expand, 3x3 stride 2 (first layer of a stage), the stem
     (32, 256, 56, 56, 64, 1, 1, 1, 1, 0), (32, 512, 28, 28, 128, 1, 1, 1, 1, 0), (32, 2048, 7, 7, 512, 1, 1, 1, 1, 0),
     (32, 1024, 14, 14, 256, 1, 1, 1, 1, 0), (32, 128, 56, 56, 128, 3, 3, 2, 2, 1), (32, 256, 28, 28, 256, 3, 3, 2, 2, 1),
-    (32, 512, 14, 14, 512, 3, 3, 2, 2, 1), (8, 3, 224, 224, 64, 7, 7, 2, 2, 3),
+    (32, 512, 14, 14, 512, 3, 3, 2, 2, 1), (8, 3, 224, 224, 64, 7, 7, 2, 2, 3), (32, 3, 224, 224, 64, 7, 7, 2, 2, 3),
+    # the 1x1 stride-2 projections (run_resnet50.sh:24,29) at batch 32 and 1; a 3x3 stride-2 layer at batch 1
+    (32, 512, 28, 28, 1024, 1, 1, 2, 2, 0), (32, 1024, 14, 14, 2048, 1, 1, 2, 2, 0),
+    (1, 512, 28, 28, 1024, 1, 1, 2, 2, 0), (1, 1024, 14, 14, 2048, 1, 1, 2, 2, 0), (1, 256, 28, 28, 256, 3, 3, 2, 2, 1),
+    (1, 128, 56, 56, 128, 3, 3, 2, 2, 1), (1, 512, 14, 14, 512, 3, 3, 2, 2, 1),
     # windows of 63, 64 (one 64-bit tap mask) and 81 taps (beyond it: the pointer gather)
     (2, 3, 20, 21, 8, 7, 9, 1, 1, 3), (1, 4, 19, 19, 9, 8, 8, 2, 2, 4), (2, 3, 20, 20, 8, 9, 9, 1, 1, 4),
+    # 81 taps with a channel count that is a whole number of stages: the pointer gather over a tap-major filter
+    (1, 16, 20, 20, 8, 9, 9, 1, 1, 4), (2, 32, 12, 14, 70, 9, 9, 2, 1, 3),
 ]
 
 
@@ -461,7 +489,7 @@ def test_implicit_gemm_input_of_2_gib_takes_the_pointer_gather(lib):
     """Inputs below 2 GiB are gathered through a buffer resource with 32-bit offsets; a larger one
     falls back to 64-bit pointers.  One tap per filter gives an exact answer at this size."""
     import fastconv_amd as F
-    N, C, H, W, K = 1, 8, 8200, 8200, 2
+    N, C, H, W, K = 1, 16, 5800, 5800, 2          # 16 channels: a whole stage, so the filter is laid out tap-major
     assert 4 * N * C * H * W >= 1 << 31
     s = O.shape(N, C, H, W, K)
     x = O.rng_uniform(5, (N, C, H, W))
