@@ -33,7 +33,7 @@ class ConvShape(C.Structure):
 
 class GemmConfig(C.Structure):
     _fields_ = [(n, C.c_int) for n in
-                ("id", "bm", "bn", "bk", "waves_m", "waves_n", "lds_bytes", "direct_lds")]
+                ("id", "bm", "bn", "bk", "waves_m", "waves_n", "lds_bytes", "waves_k")]
 
 
 class WinoPlan(C.Structure):

@@ -57,6 +57,16 @@ int fc_set_error(fc_context *ctx, int status, const char *what, hipError_t err);
 // implicit_gemm.hip: looks up the static workspace of this context's device (once per device)
 int fc_igemm_static_init(fc_context *ctx);
 bool fc_ctx_ok(const fc_context *ctx);
+// implicit_gemm_wavesplit.hip: the implicit-GEMM configurations whose workgroups split the reduction over their
+// wavefronts (small tiles, one launch per layer, for layers with few output pixels).  `index` counts them from 0;
+// their public ids follow the LDS-tiled configurations of implicit_gemm.hip.
+int fc_igemm_ws_num_shapes();
+void fc_igemm_ws_get_config(int index, int id, fc_gemm_config *cfg);
+bool fc_igemm_ws_supports(const fc_conv_shape *s);
+int fc_igemm_ws_choose(const fc_conv_shape *s, long Npix);      // index of the untuned choice, or -1
+int fc_igemm_ws_pack(fc_context *ctx, const fc_igemm_plan *plan, const float *w_dev, float *Wq_dev, int32_t *table_dev);
+int fc_igemm_ws_run(fc_context *ctx, const fc_igemm_plan *plan, int index, const float *x_dev, const float *Wq_dev,
+                    const int32_t *table_dev, const float *bias_dev, int relu, float *y_dev, bool timed);
 // wino_smallc.hip: the single-kernel Winograd path of layers with at most four input channels.
 // Called by the fc_wino_*onepass* entry points after they have checked plan and pointers.
 bool fc_wino_smallc_applies(const fc_conv_shape *s);

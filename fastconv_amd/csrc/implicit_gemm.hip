@@ -530,7 +530,7 @@ typedef IgTile<128, 256, 16, 2, 2> Ig6;
 typedef IgTile<64, 256, 16, 1, 4> Ig7;
 
 const fc_gemm_config kIgConfigs[] = {
-#define FC_CFG(id, T) {id, T::BM_, T::BN_, T::BK_, T::WGM_, T::WGN_, T::LDS_BYTES, 0}
+#define FC_CFG(id, T) {id, T::BM_, T::BN_, T::BK_, T::WGM_, T::WGN_, T::LDS_BYTES, 1}
     FC_CFG(0, Ig0), FC_CFG(1, Ig1), FC_CFG(2, Ig2), FC_CFG(3, Ig3),
     FC_CFG(4, Ig4), FC_CFG(5, Ig5), FC_CFG(6, Ig6), FC_CFG(7, Ig7),
 #undef FC_CFG
@@ -558,11 +558,13 @@ void launch(fc_context *ctx, IgemmParams &p) {
 
 }  // namespace
 
-extern "C" int fc_igemm_num_configs(void) { return kNumIgConfigs; }
+// Configuration ids: the LDS-tiled shapes of this file first, then the shapes of implicit_gemm_wavesplit.hip.
+extern "C" int fc_igemm_num_configs(void) { return kNumIgConfigs + fc_igemm_ws_num_shapes(); }
 
 extern "C" int fc_igemm_get_config(int id, fc_gemm_config *cfg) {
-    if (!cfg || id < 0 || id >= kNumIgConfigs) return FC_ERR_INVALID;
-    *cfg = kIgConfigs[id];
+    if (!cfg || id < 0 || id >= fc_igemm_num_configs()) return FC_ERR_INVALID;
+    if (id < kNumIgConfigs) *cfg = kIgConfigs[id];
+    else fc_igemm_ws_get_config(id - kNumIgConfigs, id, cfg);
     return FC_OK;
 }
 
@@ -589,6 +591,14 @@ extern "C" int fc_igemm_default_config(const fc_conv_shape *s) {
         const double cost = mp * np * kp / (kRate[id] * (0.8 + 0.2 * fill));
         if (cost < bestCost) { bestCost = cost; best = id; }
     }
+    // A layer that this tile shape can only fill the chip with by splitting the reduction over workgroups
+    // (a pass of partial sums through memory and a second launch) goes to the kernels that split it inside
+    // the workgroup instead, while it is small enough for them.
+    fc_igemm_plan plan;
+    if (fc_igemm_make_plan(s, best, &plan) == FC_OK && plan.split_k > 1) {
+        const int ws = fc_igemm_ws_choose(s, plan.Npix);
+        if (ws >= 0) return kNumIgConfigs + ws;
+    }
     return best;
 }
 
@@ -611,6 +621,13 @@ extern "C" int fc_igemm_make_plan(const fc_conv_shape *s, int config, fc_igemm_p
     plan->config = config;
     plan->Wp_bytes = sizeof(float) * (size_t)plan->Kred_pad * plan->K_pad;
     plan->table_bytes = sizeof(int32_t) * 2 * (size_t)plan->Kred_pad;
+    if (config >= kNumIgConfigs) {
+        // the reduction is split inside the workgroups: one launch, no workspace
+        if (!fc_igemm_ws_supports(s)) return FC_ERR_UNSUPPORTED;
+        plan->split_k = 1;
+        plan->ws_bytes = 0;
+        return FC_OK;
+    }
     // Small layers do not fill 256 CUs with (K_pad/BM) x (Npix/BN) workgroups: split the
     // reduction until about three workgroups per CU exist, keeping >= 4 LDS stages per part.
     const long blocks = (long)(plan->K_pad / cfg.bm) * ((npix + cfg.bn - 1) / cfg.bn);
@@ -653,6 +670,7 @@ extern "C" int fc_igemm_pack_filter(fc_context *ctx, const fc_igemm_plan *plan, 
     const fc_conv_shape &s = plan->shape;
     const dim3 grid((plan->K_pad + 63) / 64, (plan->Kred_pad + 3) / 4);
     if (grid.y > 65535) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_igemm_pack_filter: reduction too long", hipSuccess);
+    if (plan->config >= kNumIgConfigs) return fc_igemm_ws_pack(ctx, plan, w_dev, Wp_dev, table_dev);
     fc_gemm_config cfg;
     fc_igemm_get_config(plan->config, &cfg);
     const int tapMajor = s.C % cfg.bk == 0 ? 1 : 0;      // must match the kernel's choice in launch()
@@ -734,6 +752,8 @@ static int igemm_run(fc_context *ctx, const fc_igemm_plan *plan, const float *x_
     if (!x_dev || !Wp_dev || !table_dev || !y_dev) return fail(FC_ERR_INVALID, "null buffer");
     if ((uintptr_t)Wp_dev & 15) return fail(FC_ERR_INVALID, "Wp must be 16-byte aligned");
     if (plan->split_k > 1 && !ws_dev) return fail(FC_ERR_INVALID, "this plan splits the reduction and needs ws_bytes of workspace");
+    if (plan->config >= kNumIgConfigs)
+        return fc_igemm_ws_run(ctx, plan, plan->config - kNumIgConfigs, x_dev, Wp_dev, table_dev, bias_dev, relu, y_dev, timed);
     fc_gemm_config cfg;
     fc_igemm_get_config(plan->config, &cfg);
     const fc_conv_shape &s = plan->shape;

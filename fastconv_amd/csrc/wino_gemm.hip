@@ -293,7 +293,7 @@ typedef TileCfg<128, 128, 32, 2, 2> Cfg9;
 typedef TileCfg<64, 32, 16, 2, 1> Cfg10;
 
 const fc_gemm_config kConfigs[] = {
-#define FC_CFG(id, T) {id, T::BM_, T::BN_, T::BK_, T::WGM_, T::WGN_, T::LDS_BYTES, 0}
+#define FC_CFG(id, T) {id, T::BM_, T::BN_, T::BK_, T::WGM_, T::WGN_, T::LDS_BYTES, 1}
     FC_CFG(0, Cfg0), FC_CFG(1, Cfg1), FC_CFG(2, Cfg2), FC_CFG(3, Cfg3), FC_CFG(4, Cfg4), FC_CFG(5, Cfg5),
     FC_CFG(6, Cfg6), FC_CFG(7, Cfg7), FC_CFG(8, Cfg8), FC_CFG(9, Cfg9), FC_CFG(10, Cfg10),
 #undef FC_CFG

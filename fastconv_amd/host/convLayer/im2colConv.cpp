@@ -76,8 +76,8 @@ int ConvIm2colLayer::Init() {
     AllocateFor(config_best);
     fc_gemm_config c;
     fc_igemm_get_config(config, &c);
-    printf("Testing M=%d N=%ld K=%d batch=%zu tile %dx%dx%d (cfg %d) reduction split %d\n", M, N, K, batch, c.bm, c.bn,
-           c.bk, config, plan.split_k);
+    printf("Testing M=%d N=%ld K=%d batch=%zu tile %dx%dx%d (cfg %d) reduction split %d over workgroups, %d over wavefronts\n",
+           M, N, K, batch, c.bm, c.bn, c.bk, config, plan.split_k, c.waves_k);
     return 1;
 }
 
@@ -130,6 +130,8 @@ int ConvIm2colLayer::Tuning() {
     if (channel_bias) dev.SetBias(channel_bias, output_channels);
     double best_ms = 1e100;
     for (int cfg = 0; cfg < fc_igemm_num_configs(); cfg++) {
+        fc_igemm_plan probe;
+        if (fc_igemm_make_plan(&s, cfg, &probe) != FC_OK) continue;      // a tile shape that cannot run this layer
         const size_t mark = d.Mark();
         AllocateFor(cfg);
         RunOnce();
@@ -146,7 +148,8 @@ int ConvIm2colLayer::Tuning() {
             dev.Download(output_data, output_elements());
             dis = diff(output_ref, output_data, (int)output_elements());
         }
-        printf("M=%d N=%ld K=%d tile %dx%dx%d cfg=%d time=%.3f, diff=%.3f\n", M, N, K, c.bm, c.bn, c.bk, cfg, ms, dis);
+        printf("M=%d N=%ld K=%d tile %dx%dx%d waves %dx%dx%d cfg=%d time=%.3f, diff=%.3f\n", M, N, K, c.bm, c.bn, c.bk,
+               c.waves_m, c.waves_n, c.waves_k, cfg, ms, dis);
         if (ms < best_ms) {
             best_ms = ms;
             config_best = cfg;

@@ -141,13 +141,15 @@ int fc_clock_probe_end(fc_context *ctx, double *mhz, int capacity, int *n_sample
 /* Tile shapes of the batched GEMM stage.  The reference tunes
  * ocBlock/tileBlock/icBlock and a 4x4 or 4x5 register kernel
  * (convLayer/winoF63ConvZC.cpp:25-174); here a configuration is a workgroup
- * tile BM (output channels) x BN (tiles) x BK (input channels) and a wave grid. */
+ * tile BM (output channels) x BN (tiles) x BK (input channels) and a wave grid
+ * (waves_m x waves_n wavefronts side by side over the tile, times waves_k
+ * wavefronts that each take a share of the reduction). */
 typedef struct {
     int id;
     int bm, bn, bk;
     int waves_m, waves_n;
     int lds_bytes;
-    int direct_lds;           /* 1: operands go global -> LDS without passing registers */
+    int waves_k;              /* wavefronts of a workgroup that split the reduction among themselves (1: no split) */
 } fc_gemm_config;
 
 int fc_wino_gemm_num_configs(void);

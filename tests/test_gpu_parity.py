@@ -526,6 +526,84 @@ def test_implicit_gemm_every_tile_config(lib):
         assert O.max_rel_err(y, truth) <= TOL_IM2COL, cfg.id
 
 
+# every conv geometry of ResNet-50 (run_resnet50.sh:10-30 plus the 3x3 stride-2 variant): (C, K, H, kernel, stride, pad)
+RESNET50_GEOMETRIES = [
+    (3, 64, 224, 7, 2, 3), (64, 64, 56, 1, 1, 0), (64, 64, 56, 3, 1, 1), (64, 256, 56, 1, 1, 0), (256, 64, 56, 1, 1, 0),
+    (256, 128, 56, 1, 1, 0), (128, 128, 56, 3, 2, 1), (128, 128, 28, 3, 1, 1), (128, 512, 28, 1, 1, 0), (512, 128, 28, 1, 1, 0),
+    (256, 512, 56, 1, 2, 0), (512, 256, 28, 1, 1, 0), (256, 256, 28, 3, 2, 1), (256, 256, 14, 3, 1, 1), (256, 1024, 14, 1, 1, 0),
+    (1024, 256, 14, 1, 1, 0), (512, 1024, 28, 1, 2, 0), (1024, 512, 14, 1, 1, 0), (512, 512, 14, 3, 2, 1), (512, 512, 7, 3, 1, 1),
+    (512, 2048, 7, 1, 1, 0), (2048, 512, 7, 1, 1, 0), (1024, 2048, 14, 1, 2, 0),
+]
+
+
+@pytest.mark.parametrize("geo", RESNET50_GEOMETRIES)
+def test_implicit_gemm_batch1_resnet50_layers(lib, geo):
+    """Batch 1, the library's untuned choice: against the fp64 oracle at 1e-5, the same bits on a second run,
+    and (but for the layers that fill the chip unsplit) one launch with the reduction split inside the workgroups."""
+    C, K, H, ks, st, pad = geo
+    s = O.shape(1, C, H, H, K, ks, ks, st, st, pad)
+    cs = cshape(s)
+    cfg = lib.igemm_default_config(cs)
+    g = lib.igemm_configs()[cfg]
+    plan = lib.igemm_plan(cs, cfg)
+    announce("batch-1 ResNet-50 layer", geo, "tile %dx%d, %d wavefronts over the reduction, split %d" % (g.bm, g.bn, g.waves_k, plan.split_k))
+    if C % 16 == 0 and (C, K, H, ks) not in ((64, 64, 56, 1), (64, 256, 56, 1)):
+        assert g.waves_k > 1 and plan.split_k == 1 and plan.ws_bytes == 0
+    x, w = O.make_inputs(s, seed=C + K)
+    bias = O.rng_uniform(K, (K,))
+    y1 = lib.implicit_gemm_conv(cs, x, w, bias=bias, relu=True)
+    y2 = lib.implicit_gemm_conv(cs, x, w, bias=bias, relu=True)
+    assert np.array_equal(y1, y2)
+    assert O.max_rel_err(y1, np.maximum(O.naive_conv_f64(s, x, w, bias), 0.0)) <= TOL_IM2COL
+    assert O.max_rel_err(lib.implicit_gemm_conv(cs, x, w), O.naive_conv_f64(s, x, w)) <= TOL_IM2COL
+
+
+WAVESPLIT_SHAPES = [
+    # tap-major, windows inside the image (1x1, unpadded 3x3, stride 2): pixel blocks that end inside an image and span two
+    (1, 32, 7, 7, 40, 1, 1, 1, 1, 0), (3, 16, 9, 10, 33, 1, 1, 2, 2, 0), (2, 48, 11, 9, 20, 3, 3, 1, 1, 0), (1, 64, 13, 13, 64, 2, 2, 2, 2, 0),
+    # tap-major with padding (taps outside the image are refused by the buffer's range check)
+    (1, 16, 7, 7, 16, 3, 3, 1, 1, 1), (2, 32, 14, 14, 48, 3, 3, 2, 2, 1), (1, 80, 5, 6, 17, 5, 5, 1, 1, 2), (1, 16, 12, 12, 8, 7, 7, 2, 2, 3),
+    # channel counts that are not whole units: the row table
+    (2, 24, 9, 9, 30, 3, 3, 1, 1, 1), (1, 3, 20, 20, 10, 7, 7, 2, 2, 3), (3, 5, 8, 8, 70, 1, 1, 1, 1, 0), (1, 1, 6, 6, 1, 3, 3, 1, 1, 1),
+    # fewer reduction units than wavefronts; one pixel
+    (1, 16, 4, 4, 16, 1, 1, 1, 1, 0), (1, 32, 1, 1, 9, 1, 1, 1, 1, 0), (1, 16, 3, 3, 5, 3, 3, 1, 1, 0),
+]
+
+
+@pytest.mark.parametrize("shp", WAVESPLIT_SHAPES)
+def test_implicit_gemm_reduction_split_inside_the_workgroup(lib, shp):
+    """Every configuration of the kernels that split the reduction over the wavefronts of a workgroup, with
+    bias and ReLU, against the fp64 oracle."""
+    s = O.shape(*shp)
+    x, w = O.make_inputs(s, seed=shp[1] + 3 * shp[4])
+    bias = O.rng_uniform(6, (s.K,))
+    truth = np.maximum(O.naive_conv_f64(s, x, w, bias), 0.0)
+    n = 0
+    for cfg in lib.igemm_configs():
+        if cfg.waves_k == 1:
+            continue
+        announce("wavefront-split reduction", shp, "tile %dx%d, %d wavefronts" % (cfg.bm, cfg.bn, cfg.waves_k))
+        plan = lib.igemm_plan(cshape(s), cfg.id)
+        assert plan.split_k == 1 and plan.ws_bytes == 0
+        y = lib.implicit_gemm_conv(cshape(s), x, w, bias=bias, relu=True, config=cfg.id)
+        assert y.shape == truth.shape
+        assert O.max_rel_err(y, truth) <= TOL_IM2COL, cfg.id
+        n += 1
+    assert n >= 12
+
+
+def test_implicit_gemm_wavefront_split_refuses_what_it_cannot_address(lib):
+    """These kernels address x with one 32-bit offset (bit 31 spare) and one 64-bit mask of taps: larger layers
+    are refused at plan time and the untuned choice stays with the LDS-tiled kernels."""
+    import fastconv_amd as F
+    ws = [c.id for c in lib.igemm_configs() if c.waves_k > 1]
+    for bad in [O.shape(1, 16, 5800, 5800, 2), O.shape(2, 3, 20, 20, 8, 9, 9, 1, 1, 4)]:
+        with pytest.raises(F.FastConvError) as e:
+            lib.igemm_plan(cshape(bad), ws[0])
+        assert e.value.status == -6
+        assert lib.igemm_configs()[lib.igemm_default_config(cshape(bad))].waves_k == 1
+
+
 def test_implicit_gemm_full_tile_epilogue_paths(lib):
     """Output-channel counts that are whole tiles take the predicate-free epilogue (plain, and
     with bias / ReLU); pixel blocks that straddle images and end inside a block are part of it."""
@@ -546,18 +624,19 @@ def test_implicit_gemm_full_tile_epilogue_paths(lib):
 
 
 def test_implicit_gemm_split_reduction_is_exact_and_repeatable(lib):
-    """Batch-1 layers are too small to fill the GPU: their reduction is split and the parts
-    are added in a fixed order, so two runs give the same bits."""
+    """Under the LDS-tiled 64x64 shape batch-1 layers are too few workgroups to fill the GPU: their
+    reduction is split over workgroups and the parts are added in a fixed order by a second kernel, so
+    two runs give the same bits."""
     for shp in [(1, 2048, 7, 7, 512, 1, 1, 1, 1, 0), (1, 256, 56, 56, 256, 3, 3, 1, 1, 1),
                 (1, 512, 14, 14, 512, 3, 3, 2, 2, 1), (1, 1024, 14, 14, 256, 1, 1, 1, 1, 0)]:
         s = O.shape(*shp)
-        plan = lib.igemm_plan(cshape(s), lib.igemm_default_config(cshape(s)))
+        plan = lib.igemm_plan(cshape(s), 3)
         assert plan.split_k > 1, shp
         x, w = O.make_inputs(s, seed=3)
         bias = O.rng_uniform(9, (s.K,))
         announce("split reduction", shp, "parts", plan.split_k)
-        y1 = lib.implicit_gemm_conv(cshape(s), x, w, bias=bias, relu=True)
-        y2 = lib.implicit_gemm_conv(cshape(s), x, w, bias=bias, relu=True)
+        y1 = lib.implicit_gemm_conv(cshape(s), x, w, bias=bias, relu=True, config=3)
+        y2 = lib.implicit_gemm_conv(cshape(s), x, w, bias=bias, relu=True, config=3)
         assert np.array_equal(y1, y2)
         truth = np.maximum(O.naive_conv_f64(s, x, w, bias), 0.0)
         assert O.max_rel_err(y1, truth) <= TOL_IM2COL
