@@ -320,9 +320,12 @@ def copy_probe(mib):
 
 def measured_traffic():
     """{(kernel, N, C, K, H, ks, st, 'BMxBNxBK'): bytes per launch} parsed from the committed rocprofv3 counter
-    summary; empty when the file is absent (`traffic` is then null)."""
+    summary; empty when the file is absent or was taken with other kernel sources than this tree's
+    (`traffic` is then null)."""
     out = {}
-    if not os.path.exists(TRAFFIC_PROFILE):
+    from fastconv_amd import provenance
+    # the file names the kernel sources it was measured on: once they have changed its numbers describe other code
+    if not os.path.exists(TRAFFIC_PROFILE) or not provenance.sources_current(TRAFFIC_PROFILE):
         return out
     pat = re.compile(r"^traffic kernel=(\w+) N=(\d+) C=(\d+) K=(\d+) H=(\d+) ks=(\d+) st=(\d+) tile=(\w+) "
                      r".*measured_bytes=(\d+)")
@@ -391,16 +394,17 @@ def run_workload(name, steps, warmup, o, detail=True, offline_filter=None):
             lay.set_blocks(L, cfg, ib if pipe == "fused" else N)
             L.wino_filter_transform(lay.plan, lay.w, lay.U)
             g = L.wino_configs()[cfg]
-            log("layer %s: winograd %s, tile %dx%dx%d (cfg %d) %.3f ms%s"
-                % (lay.name(), pipe, g.bm, g.bn, g.bk, cfg, ms, " (im2col %.3f ms)" % ires[1] if ires else ""))
+            log("layer %s: winograd %s, tile %dx%dx%d (cfg %d)%s"
+                % (lay.name(), pipe, g.bm, g.bn, g.bk, cfg,
+                   " %.3f ms%s" % (ms, " (im2col %.3f ms)" % ires[1] if ires else "") if tune else ", the library's untuned choice"))
         else:
             cfg, ms = ires
             lay.algo = "im2col"
             lay.setup_im2col(L, cfg)
             g = L.igemm_configs()[cfg]
-            log("layer %s: im2col, tile %dx%dx%d (cfg %d) split %d %.3f ms%s"
-                % (lay.name(), g.bm, g.bn, g.bk, cfg, lay.iplan.split_k, ms,
-                   " (winograd %.3f ms)" % wres[2] if wres else ""))
+            log("layer %s: im2col, tile %dx%dx%d (cfg %d), reduction split %d over workgroups, %d over wavefronts%s"
+                % (lay.name(), g.bm, g.bn, g.bk, cfg, lay.iplan.split_k, g.waves_k,
+                   " %.3f ms%s" % (ms, " (winograd %.3f ms)" % wres[2] if wres else "") if tune else ", the library's untuned choice"))
     L.sync()
 
     filter_ready = o.offline_filter if offline_filter is None else offline_filter
@@ -597,7 +601,11 @@ def run_workload(name, steps, warmup, o, detail=True, offline_filter=None):
         tr = None
         if all(k in traffic for k in keys):
             tr = round(sum(traffic[k] * l.repeats for k, l in zip(keys, il)) / sum(l.repeats for l in il))
-        roofline = dict(transforms["implicit_gemm"], kernel="igemm_conv_kernel", traffic=tr,
+        n_ws = sum(l.repeats for l in il if L.igemm_configs()[l.iplan.config].waves_k > 1)
+        n_all = sum(l.repeats for l in il)
+        kname = ("igemm_conv_kernel" if n_ws == 0 else "igemm_wavesplit_kernel" if n_ws == n_all else
+                 "igemm_wavesplit_kernel (%d of %d launches per step), igemm_conv_kernel" % (n_ws, n_all))
+        roofline = dict(transforms["implicit_gemm"], kernel=kname, traffic=tr,
                         avg_launch_ms=round(igemm_stage[0] / igemm_stage[1], 5))
         if shader_clock:
             at_clock = info["compute_units"] * 256 * shader_clock["mean_mhz"] * 1e6 / 1e12
@@ -675,6 +683,7 @@ def run_workload(name, steps, warmup, o, detail=True, offline_filter=None):
         if lay.algo == "im2col":
             ms = L.stage_time(ST_IGEMM)[0] / reps
             row.update(ms=round(ms, 4), gflops=round(lay.flops / (ms * 1e-3) / 1e9, 1), split_k=lay.iplan.split_k,
+                       waves_over_reduction=g.waves_k,
                        gemm_tflops=round(lay.flops / (ms * 1e-3) / 1e12, 2),
                        gemm_frac_mfma=round(lay.flops / (ms * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 3))
         else:
@@ -752,7 +761,7 @@ def run_workload(name, steps, warmup, o, detail=True, offline_filter=None):
 
     roofline["events"] = ("inside the timed region" if stage_events in ("gemm", "all") and not o.graph
                           else "in the untimed steps after it")
-    if roofline.get("kernel") == "igemm_conv_kernel" and igemm_events:
+    if str(roofline.get("kernel", "")).startswith("igemm_") and igemm_events:
         roofline["events"] = igemm_events
     out = {
         "metric": "effective GFLOP/s over the conv stack (direct-conv FLOP count / time)",

@@ -252,7 +252,8 @@ struct WsShape {
 };
 // the configurations after the LDS-tiled ones of implicit_gemm.hip, in the order of their ids
 const WsShape kWsShapes[] = {{1, 1, 4}, {1, 1, 8}, {1, 1, 16}, {1, 2, 4}, {1, 2, 8}, {1, 2, 16},
-                             {2, 1, 4}, {2, 1, 8}, {2, 1, 16}, {2, 2, 4}, {2, 2, 8}, {2, 2, 16}};
+                             {2, 1, 4}, {2, 1, 8}, {2, 1, 16}, {2, 2, 4}, {2, 2, 8}, {2, 2, 16},
+                             {4, 2, 4}, {4, 2, 8}, {2, 4, 4}, {2, 4, 8}, {4, 4, 4}};
 const int kNumWsShapes = sizeof(kWsShapes) / sizeof(kWsShapes[0]);
 
 template <int MT, int NT, int NW>
@@ -281,9 +282,9 @@ void fc_igemm_ws_get_config(int index, int id, fc_gemm_config *cfg) {
 
 // These kernels gather through a buffer resource with 32-bit offsets (bit 31 to spare) and one 64-bit mask of taps
 bool fc_igemm_ws_supports(const fc_conv_shape *s) {
-    // (the filter is addressed the same way: K rounded up to 32 at most)
+    // (the filter is addressed the same way: K rounded up to 64 at most)
     return 4.0 * s->N * s->C * s->H * s->W < 2147483648.0 && s->kh * s->kw <= 64 &&
-           4.0 * (s->K + 31.0) * ((double)s->C * s->kh * s->kw + 15.0) < 2147483648.0;
+           4.0 * (s->K + 63.0) * ((double)s->C * s->kh * s->kw + 15.0) < 2147483648.0;
 }
 
 // Untuned choice among these configurations, for a layer whose reduction the LDS-tiled kernels would have to
@@ -354,6 +355,7 @@ int fc_igemm_ws_run(fc_context *ctx, const fc_igemm_plan *plan, int index, const
         FC_WS_CASE(3, 1, 2, 4); FC_WS_CASE(4, 1, 2, 8); FC_WS_CASE(5, 1, 2, 16);
         FC_WS_CASE(6, 2, 1, 4); FC_WS_CASE(7, 2, 1, 8); FC_WS_CASE(8, 2, 1, 16);
         FC_WS_CASE(9, 2, 2, 4); FC_WS_CASE(10, 2, 2, 8); FC_WS_CASE(11, 2, 2, 16);
+        FC_WS_CASE(12, 4, 2, 4); FC_WS_CASE(13, 4, 2, 8); FC_WS_CASE(14, 2, 4, 4); FC_WS_CASE(15, 2, 4, 8); FC_WS_CASE(16, 4, 4, 4);
         default: return fc_set_error(ctx, FC_ERR_INVALID, "fc_conv_implicit_gemm: unknown tile configuration", hipSuccess);
     }
 #undef FC_WS_CASE

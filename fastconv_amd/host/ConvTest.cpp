@@ -434,18 +434,46 @@ int main(int argc, char *argv[]) {
             if (!ok && options.strict) status = 2;
         }
         if (options.json) {
+            // Each stage against the roofline that bounds it (MI355X: 157.3 TFLOP/s of fp32 MFMA, 8 TB/s of HBM),
+            // from the algorithmic work of the stage: Winograd products 2*64*K*C*T flop over T = N*ceil(OH/6)*ceil(OW/6)
+            // tiles (the implicit GEMM: the direct-convolution count), input transform x once + V once, output
+            // transform M once + y once, filter transform w once + U once.
+            const double kPeakTflops = 157.3, kPeakGbs = 8000.0;
+            const bool wino = options.algorithm == nnp_convolution_algorithm_winograd;
+            const double N = (double)options.batch, C = (double)input_channels, K = (double)output_channels;
+            const double T = N * (double)((output_size.height + 5) / 6) * (double)((output_size.width + 5) / 6);
+            const double gemm_flops = wino ? 2.0 * 64.0 * K * C * T : conv_test->flops();
+            const double it_bytes = 4.0 * N * C * (double)input_size.height * (double)input_size.width + 256.0 * C * T;
+            const double ot_bytes = 256.0 * K * T + 4.0 * N * K * (double)output_size.height * (double)output_size.width;
+            const double kt_bytes = 4.0 * K * C * (9.0 + 64.0);
+            char roof[512];
+            int at = 0;
+            auto field = [&](const char *name, double work, double stage, double unit, double peak, const char *frac_name) {
+                if (stage > 0.0) {
+                    const double rate = work / (stage * 1e-3) / unit;
+                    at += snprintf(roof + at, sizeof roof - at, ", \"%s\": %.2f, \"%s\": %.4f", name, rate, frac_name, rate / peak);
+                } else {
+                    at += snprintf(roof + at, sizeof roof - at, ", \"%s\": null, \"%s\": null", name, frac_name);
+                }
+            };
+            field("gemm_tflops", gemm_flops, stage_ms[2], 1e12, kPeakTflops, "gemm_frac_mfma");
+            field("input_tran_gbs", it_bytes, wino ? stage_ms[0] : 0.0, 1e9, kPeakGbs, "input_tran_frac_hbm");
+            field("output_tran_gbs", ot_bytes, wino ? stage_ms[3] : 0.0, 1e9, kPeakGbs, "output_tran_frac_hbm");
+            field("kernel_tran_gbs", kt_bytes, wino ? stage_ms[1] : 0.0, 1e9, kPeakGbs, "kernel_tran_frac_hbm");
             printf("{\"algorithm\": \"%s%s\", \"batch\": %zu, \"ic\": %zu, \"oc\": %zu, \"ih\": %zu, \"iw\": %zu, "
                    "\"kh\": %zu, \"kw\": %zu, \"stride\": %zu, \"pad\": %zu, \"config\": %d, \"ms\": %.6f, "
                    "\"gflops\": %.2f, \"input_tran_ms\": %.6f, \"kernel_tran_ms\": %.6f, \"gemm_ms\": %.6f, "
                    "\"output_tran_ms\": %.6f, \"max_rel_err\": %.4e, \"naive_ms\": %.3f, \"naive_threads\": %zu, "
-                   "\"checked_images\": %zu, \"images_per_block\": %d, \"kernel_transform\": \"%s\"}\n",
+                   "\"checked_images\": %zu, \"images_per_block\": %d, \"kernel_transform\": \"%s\"%s, "
+                   "\"peak_mfma_tflops\": %.1f, \"peak_hbm_gbs\": %.0f}\n",
                    algorithm_name(options.algorithm),
                    (options.algorithm == nnp_convolution_algorithm_winograd && options.blocked_variant) ? "_blocked" : "",
                    options.batch, input_channels, output_channels, input_size.height, input_size.width,
                    kernel_size.height, kernel_size.width, output_subsampling.height, options.input_padding,
                    chosen_config, ms, gflops, stage_ms[0], stage_ms[1], stage_ms[2], stage_ms[3], err, naive_ms,
                    options.threads, options.check ? checked : (size_t)0, chosen_option,
-                   kernel_transform_offline < 0 ? "n/a" : kernel_transform_offline ? "offline" : "online");
+                   kernel_transform_offline < 0 ? "n/a" : kernel_transform_offline ? "offline" : "online", roof,
+                   kPeakTflops, kPeakGbs);
         }
     }
     delete conv_test;

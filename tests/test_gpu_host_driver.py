@@ -55,6 +55,25 @@ def _json_line(out):
     return json.loads([l for l in out.splitlines() if l.startswith("{")][-1])
 
 
+def test_json_line_reports_every_stage_against_its_roofline():
+    """conv_test --json: per-stage rates and their fraction of the fp32 MFMA peak (GEMM stages) or of the HBM
+    peak (transforms), consistent with the stage times on the same line."""
+    base = [_exe("conv_test"), "-ic", "128", "-oc", "128", "-is", "56", "56", "-ks", "3", "3", "-ip", "1", "-n", "8",
+            "-i", "5", "-t", "16", "--check-images", "1", "--strict", "--json"]
+    j = _json_line(_run(base + ["-a", "winograd", "--variant", "zc"]))
+    assert j["peak_mfma_tflops"] == 157.3 and j["peak_hbm_gbs"] == 8000
+    T = 8 * 10 * 10
+    assert j["gemm_tflops"] == pytest.approx(2 * 64 * 128 * 128 * T / (j["gemm_ms"] * 1e-3) / 1e12, rel=1e-2)
+    assert j["gemm_frac_mfma"] == pytest.approx(j["gemm_tflops"] / 157.3, abs=2e-4)
+    assert j["input_tran_gbs"] == pytest.approx((4 * 8 * 128 * 56 * 56 + 256 * 128 * T) / (j["input_tran_ms"] * 1e-3) / 1e9, rel=1e-2)
+    assert j["output_tran_gbs"] == pytest.approx((256 * 128 * T + 4 * 8 * 128 * 56 * 56) / (j["output_tran_ms"] * 1e-3) / 1e9, rel=1e-2)
+    for k in ("gemm_frac_mfma", "input_tran_frac_hbm", "output_tran_frac_hbm"):
+        assert 0.0 < j[k] < 1.0, k
+    j = _json_line(_run(base + ["-a", "im2col"]))
+    assert j["gemm_tflops"] == pytest.approx(2 * 8 * 128 * 128 * 56 * 56 * 9 / (j["gemm_ms"] * 1e-3) / 1e12, rel=1e-2)
+    assert 0.0 < j["gemm_frac_mfma"] < 1.0 and j["input_tran_gbs"] is None and j["output_tran_frac_hbm"] is None
+
+
 @pytest.mark.parametrize("variant", ["zc", "blocked"])
 @pytest.mark.parametrize("batch,C,H", [(64, 256, 56), (128, 256, 56), (64, 512, 28), (128, 512, 28), (64, 512, 14),
                                        (128, 512, 14)])
