@@ -596,8 +596,12 @@ def run_workload(name, steps, warmup, o, detail=True, offline_filter=None):
     if igemm_stage[1] > 0 and (not staged or igemm_stage[0] > stage[ST_GEMM][0]):
         wino_gemm_line = roofline if staged and stage[ST_GEMM][1] > 0 else None
         il = [l for l in layers if l.algo == "im2col"]
-        keys = [("igemm_conv_kernel", N, l.C, l.K, l.H, l.ks, l.st, tile_name(L.igemm_configs()[l.iplan.config]))
-                for l in il]
+        def ig_key(l):
+            g = L.igemm_configs()[l.iplan.config]
+            if g.waves_k > 1:
+                return ("igemm_wavesplit_kernel", N, l.C, l.K, l.H, l.ks, l.st, "%dx%dx%dw%d" % (g.bm, g.bn, g.bk, g.waves_k))
+            return ("igemm_conv_kernel", N, l.C, l.K, l.H, l.ks, l.st, tile_name(g))
+        keys = [ig_key(l) for l in il]
         tr = None
         if all(k in traffic for k in keys):
             tr = round(sum(traffic[k] * l.repeats for k, l in zip(keys, il)) / sum(l.repeats for l in il))
