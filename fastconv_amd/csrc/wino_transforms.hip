@@ -194,6 +194,41 @@ __device__ __forceinline__ void input_transform_block(const InTParams &p, int bx
     }
     __syncthreads();
 
+#ifdef FC_IT_VEC4
+    if (TPB == 128) {
+        // Pass 2, 16 bytes per plane store: thread = (row i of the tile, group of 4 consecutive tiles); B along the row
+        // of each of its tiles, then one 16-byte store per column frequency: 32 lanes cover the 512 bytes a block owns
+        // of a plane.
+        typedef float floatx4 __attribute__((ext_vector_type(4)));
+        const int g = tid & 31, i = tid >> 5;
+        floatx4 o[8];
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+            const uint32_t t = t0 + 4 * g + q4;
+            float r[8];
+#pragma unroll
+            for (int jj = 0; jj < 8; jj++) r[jj] = 0.f;
+            if (c < p.C && t < (uint32_t)p.T) {
+                const uint32_t gb = fc_div(t, p.divTW);
+                const int q = t - gb * p.tW, j = gb - gb0;
+                const float *row = lds + (j * 8 + i) * p.LW + q * 6;
+                float d[8];
+#pragma unroll
+                for (int jj = 0; jj < 8; jj++) d[jj] = row[jj];
+                bt8(d, r);
+            }
+#pragma unroll
+            for (int jj = 0; jj < 8; jj++) o[jj][q4] = r[jj];
+        }
+        float *pf = p.V + (size_t)(i * 8) * plane + (size_t)c * p.T_pad + t0 + 4 * g;
+#pragma unroll
+        for (int jj = 0; jj < 8; jj++) {
+            *reinterpret_cast<floatx4 *>(pf) = o[jj];
+            pf += plane;
+        }
+        return;
+    }
+#endif
     constexpr int IPT = 8 * TPB / 256;     // rows of the 8x8 tile per thread
     const int tl = tid % TPB;
     // rows ig*IPT .. +IPT-1 of the tile: the same for a whole wavefront when TPB is a multiple of 64
@@ -276,8 +311,11 @@ struct OutTParams {
 // Everything that does not depend on the lane (plane bases, band geometry of the
 // copy loop) is kept in scalar registers: the kernel spends a quarter of its
 // vector instructions on addresses otherwise.
-template <int TPB>
-__global__ __launch_bounds__(TPB) void wino_output_transform_kernel(const OutTParams p) {
+// TPT: tiles per thread.  1: a lane owns one tile and loads 4 bytes per plane.  2 (a measured variant, built
+// with -DFC_OT_VEC2): a lane owns two consecutive tiles and loads 8 bytes per plane, half the load instructions
+// per byte for 128 more registers.
+template <int TPB, int TPT = 1>
+__global__ __launch_bounds__(TPB / TPT) void wino_output_transform_kernel(const OutTParams p) {
     extern __shared__ __attribute__((aligned(16))) float lds[];   // [bands][6][OW]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -290,56 +328,68 @@ __global__ __launch_bounds__(TPB) void wino_output_transform_kernel(const OutTPa
     const int NB = (int)(gbL - gb0) + 1;
     const int bandElems = 6 * p.OW;
 
-    const uint32_t t = t0 + tid;
-    if (t <= tLast) {
-        const uint32_t gb = fc_div(t, p.divTW);
-        const int q = t - gb * p.tW, j = gb - gb0;
+    const uint32_t tFirst = t0 + TPT * tid;
+    if (tFirst <= tLast) {
         const size_t plane = (size_t)p.K_pad * p.T_pad;
         const float *src = p.M + (size_t)k * p.T_pad + t0;      // uniform
-        const uint32_t laneOff = (uint32_t)tid * 4u;
-        float m[8][8];
+        const uint32_t laneOff = (uint32_t)tid * (4u * TPT);
+        float m[TPT][8][8];
         const float *pf = src;      // stepped, not multiplied: a 64-bit product would be made with vector instructions
 #pragma unroll
         for (int f = 0; f < 64; f++) {
-            m[f >> 3][f & 7] = load_m_at(pf, laneOff);
+            if (TPT == 1) {
+                m[0][f >> 3][f & 7] = load_m_at(pf, laneOff);
+            } else {
+                typedef float floatx2 __attribute__((ext_vector_type(2)));
+                const floatx2 v = __builtin_nontemporal_load(reinterpret_cast<const floatx2 *>(reinterpret_cast<const char *>(pf) + laneOff));
+                m[0][f >> 3][f & 7] = v[0];
+                m[TPT - 1][f >> 3][f & 7] = v[1];
+            }
             pf += plane;
-        }
-        float tmp[6][8];
-#pragma unroll
-        for (int jj = 0; jj < 8; jj++) {
-            const float col[8] = {m[0][jj], m[1][jj], m[2][jj], m[3][jj], m[4][jj], m[5][jj], m[6][jj], m[7][jj]};
-            float s[6];
-            at6(col, s);
-#pragma unroll
-            for (int i = 0; i < 6; i++) tmp[i][jj] = s[i];
         }
         const float b = p.bias ? p.bias[k] : 0.f;
         // ReLU as a maximum with 0, no ReLU as a maximum with -inf: one v_maximum3_f32 either way, which keeps a NaN
         const float floorv = p.relu ? 0.f : -__builtin_inff();
-        float *img = lds + j * bandElems + q * 6;
-        const int colsLeft = p.OW - q * 6;      // columns of this tile inside the image
 #pragma unroll
-        for (int i = 0; i < 6; i++) {
-            // the bias goes in with element 1: at6 adds it (as m1 + m2 or m1 - m2) to each of its six outputs once
-            const float row[8] = {tmp[i][0], tmp[i][1] + b, tmp[i][2], tmp[i][3], tmp[i][4], tmp[i][5], tmp[i][6], tmp[i][7]};
-            float s[6];
-            at6(row, s);
+        for (int u = 0; u < TPT; u++) {
+            const uint32_t t = tFirst + u;
+            if (t > tLast) break;
+            const uint32_t gb = fc_div(t, p.divTW);
+            const int q = t - gb * p.tW, j = gb - gb0;
+            float tmp[6][8];
 #pragma unroll
-            for (int jj = 0; jj < 6; jj++) s[jj] = __builtin_elementwise_maximum(s[jj], floorv);
-            float *dstl = img + i * p.OW;
-            if (colsLeft >= 6) {
+            for (int jj = 0; jj < 8; jj++) {
+                const float col[8] = {m[u][0][jj], m[u][1][jj], m[u][2][jj], m[u][3][jj], m[u][4][jj], m[u][5][jj], m[u][6][jj], m[u][7][jj]};
+                float s[6];
+                at6(col, s);
 #pragma unroll
-                for (int jj = 0; jj < 6; jj++) dstl[jj] = s[jj];
-            } else {
+                for (int i = 0; i < 6; i++) tmp[i][jj] = s[i];
+            }
+            float *img = lds + j * bandElems + q * 6;
+            const int colsLeft = p.OW - q * 6;      // columns of this tile inside the image
 #pragma unroll
-                for (int jj = 0; jj < 6; jj++)
-                    if (jj < colsLeft) dstl[jj] = s[jj];
+            for (int i = 0; i < 6; i++) {
+                // the bias goes in with element 1: at6 adds it (as m1 + m2 or m1 - m2) to each of its six outputs once
+                const float row[8] = {tmp[i][0], tmp[i][1] + b, tmp[i][2], tmp[i][3], tmp[i][4], tmp[i][5], tmp[i][6], tmp[i][7]};
+                float s[6];
+                at6(row, s);
+#pragma unroll
+                for (int jj = 0; jj < 6; jj++) s[jj] = __builtin_elementwise_maximum(s[jj], floorv);
+                float *dstl = img + i * p.OW;
+                if (colsLeft >= 6) {
+#pragma unroll
+                    for (int jj = 0; jj < 6; jj++) dstl[jj] = s[jj];
+                } else {
+#pragma unroll
+                    for (int jj = 0; jj < 6; jj++)
+                        if (jj < colsLeft) dstl[jj] = s[jj];
+                }
             }
         }
     }
     __syncthreads();
 
-    constexpr int WAVES = TPB / 64;
+    constexpr int WAVES = TPB / TPT / 64;
     const bool vec4 = (p.OW & 3) == 0;
     const size_t chan = (size_t)p.OH * p.OW;
     for (int j = wave; j < NB; j += WAVES) {       // j and everything derived from it is uniform
@@ -555,7 +605,11 @@ extern "C" int fc_wino_output_transform(fc_context *ctx, const fc_wino_plan *pla
     if (grid.y > 65535) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_output_transform: more than 65535 channels", hipSuccess);
     if (((uintptr_t)y_dev & 15) != 0) return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_output_transform: y must be 16-byte aligned", hipSuccess);
     fc_stage_scope scope(ctx, FC_STAGE_OUTPUT_TRAN);
+#ifdef FC_OT_VEC2
+    if (tpb == 128) wino_output_transform_kernel<128, 2><<<grid, dim3(64), ldsBytes, ctx->stream>>>(p);
+#else
     if (tpb == 128) wino_output_transform_kernel<128><<<grid, dim3(128), ldsBytes, ctx->stream>>>(p);
+#endif
     else wino_output_transform_kernel<64><<<grid, dim3(64), ldsBytes, ctx->stream>>>(p);
     FC_LAUNCH_CHECK(ctx, "wino_output_transform_kernel");
     return FC_OK;
