@@ -289,23 +289,30 @@ bool fc_igemm_ws_supports(const fc_conv_shape *s) {
 
 // Untuned choice among these configurations, for a layer whose reduction the LDS-tiled kernels would have to
 // split over workgroups; -1 when they should keep the layer.  Read off per-configuration times of the
-// ResNet-50 and VGG-16 layers at batch 1 to 16 on MI355X: the largest tile that still gives 192 workgroups
-// (the tile sets how many operand loads a product costs, the workgroup count how much of the chip works);
+// ResNet-50 and VGG-16 layers at batch 1 to 32 and of a dozen other shapes on MI355X.  What a workgroup costs
+// is vector-memory instruction issue (MT + 4*NT loads per unit whatever their width), so the largest tile
+// that still spreads over the chip wins (64x32 from 768 workgroups on, 32x32 and 32x16 from 128, else 16x16),
+// unless a smaller one pads the layer less.
 // 8 wavefronts over the reduction, 4 when it is shorter than 16 units, 16 when it is long (128 units and
-// more) and the layer has at least 256 pixels.  Beyond about 4 GFLOP (2 GFLOP for strided layers, whose
-// gathered rows use half of every cache line) the LDS-tiled kernels win despite their second launch.
+// more) and the layer has at least 256 pixels.  Beyond about 8 GFLOP (2 GFLOP for strided layers, whose
+// gathered rows use half of every cache line) the LDS-tiled kernels are level or ahead despite their second launch.
 int fc_igemm_ws_choose(const fc_conv_shape *s, long Npix) {
-    if (!fc_igemm_ws_supports(s) || s->C % 16 != 0) return -1;
+    if (!fc_igemm_ws_supports(s)) return -1;
     const double flops = 2.0 * Npix * s->K * (double)s->C * s->kh * s->kw;
-    if (flops > (s->sh > 1 || s->sw > 1 ? 2.0e9 : 4.0e9)) return -1;
-    const int nUnits = s->C * s->kh * s->kw / 16;
+    if (flops > (s->sh > 1 || s->sw > 1 ? 2.0e9 : 8.0e9)) return -1;
+    const int nUnits = (s->C * s->kh * s->kw + 15) / 16;
+    // among the tiles that bring enough workgroups, the least padded work, weighted by what a product costs in loads
+    static const struct { int mt, nt; long minWgs; double weight; } kTiles[4] = {{4, 2, 768, 1.00}, {2, 2, 128, 1.15}, {2, 1, 128, 1.30}, {1, 1, 0, 1.70}};
     int mt = 1, nt = 1;
-    static const int kTiles[2][2] = {{2, 2}, {2, 1}};
-    for (int i = 0; i < 2; i++) {
-        const long wgs = (long)((s->K + 16 * kTiles[i][0] - 1) / (16 * kTiles[i][0])) * ((Npix + 16 * kTiles[i][1] - 1) / (16 * kTiles[i][1]));
-        if (wgs >= 192) { mt = kTiles[i][0]; nt = kTiles[i][1]; break; }
+    double bestCost = 1e300;
+    for (int i = 0; i < 4; i++) {
+        const long kBlocks = (s->K + 16 * kTiles[i].mt - 1) / (16 * kTiles[i].mt), pBlocks = (Npix + 16 * kTiles[i].nt - 1) / (16 * kTiles[i].nt);
+        if (kBlocks * pBlocks < kTiles[i].minWgs) continue;
+        const double cost = (double)(kBlocks * 16 * kTiles[i].mt) * (double)(pBlocks * 16 * kTiles[i].nt) * kTiles[i].weight;
+        if (cost < bestCost) { bestCost = cost; mt = kTiles[i].mt; nt = kTiles[i].nt; }
     }
-    const int nw = nUnits >= 128 && Npix >= 256 ? 16 : nUnits >= 16 ? 8 : 4;
+    int nw = nUnits >= 128 && Npix >= 256 ? 16 : nUnits >= 16 ? 8 : 4;
+    if (mt == 4 && nw == 16) nw = 8;      // no 16-wavefront 64x32 configuration: its partial tiles would not fit 64 KB of LDS
     for (int i = 0; i < kNumWsShapes; i++)
         if (kWsShapes[i].mt == mt && kWsShapes[i].nt == nt && kWsShapes[i].nw == nw) return i;
     return -1;

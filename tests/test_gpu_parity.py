@@ -879,3 +879,69 @@ def test_filter_and_input_transform_in_one_launch_match_the_two_launches(lib):
             assert np.array_equal(lib.download(U1, ushape), lib.download(U2, ushape))
             assert np.array_equal(lib.download(V1, vshape), lib.download(V2, vshape))
             lib.release(mark)
+
+
+# ------------------------------------------ untuned choices away from the layers they were fitted on
+
+def _launch_us(lib, fn, iters=20, rounds=3):
+    import time
+    fn()
+    lib.sync()
+    best = 1e30
+    for _ in range(rounds):
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            fn()
+        lib.sync()
+        best = min(best, (time.perf_counter() - t0) / iters * 1e6)
+    return best
+
+
+@pytest.mark.parametrize("geo", [
+    (8, 96, 35, 35, 192, 3, 1, 1), (32, 160, 17, 17, 160, 3, 1, 1), (4, 48, 112, 112, 48, 3, 1, 1),
+    (16, 320, 28, 28, 64, 1, 1, 0), (8, 96, 57, 57, 96, 3, 2, 1),
+])
+def test_untuned_tile_choice_is_close_to_the_best_of_a_search(lib, geo):
+    """Shapes that none of the default rules was fitted on: the configuration the library picks without tuning
+    (fc_wino_gemm_default_config for the staged Winograd pipeline, fc_igemm_default_config for the implicit GEMM)
+    takes at most 10 % longer than the best configuration of a search over all of them (20 launches back to back,
+    best of three rounds)."""
+    N, C, H, W, K, ks, st, pad = geo
+    s = O.shape(N, C, H, W, K, ks, ks, st, st, pad)
+    cs = cshape(s)
+    x, w = O.make_inputs(s, seed=1)
+    mark = lib.mark()
+    try:
+        dx, dw = lib.upload(x), lib.upload(w)
+        oh, ow = O.out_hw(s)
+        y = lib.alloc(4 * N * K * oh * ow)
+        if ks == 3 and st == 1:
+            times = {}
+            for g in lib.wino_configs():
+                plan = lib.wino_plan(cs, g.id)
+                if plan.K_pad > 2 * K and g.bm > 32:
+                    continue
+                m2 = lib.mark()
+                U, V, M = lib.alloc(plan.U_bytes), lib.alloc(plan.V_bytes), lib.alloc(plan.M_bytes)
+                times[g.id] = _launch_us(lib, lambda: lib.wino_forward(plan, dx, dw, U, V, M, y))
+                lib.release(m2)
+            d = lib.wino_default_config(cs)
+            announce("winograd", geo, "untuned config", d, "%.1f us" % times[d], "best", min(times, key=times.get), "%.1f us" % min(times.values()))
+            assert times[d] <= 1.10 * min(times.values()), (geo, times)
+        times = {}
+        for g in lib.igemm_configs():
+            try:
+                plan = lib.igemm_plan(cs, g.id)
+            except Exception:
+                continue
+            m2 = lib.mark()
+            Wp, tab = lib.alloc(plan.Wp_bytes), lib.alloc(plan.table_bytes)
+            ws = lib.alloc(plan.ws_bytes) if plan.ws_bytes else None
+            lib.igemm_pack_filter(plan, dw, Wp, tab)
+            times[g.id] = _launch_us(lib, lambda: lib.conv_implicit_gemm(plan, dx, Wp, tab, y, ws=ws))
+            lib.release(m2)
+        d = lib.igemm_default_config(cs)
+        announce("implicit gemm", geo, "untuned config", d, "%.1f us" % times[d], "best", min(times, key=times.get), "%.1f us" % min(times.values()))
+        assert times[d] <= 1.10 * min(times.values()), (geo, times)
+    finally:
+        lib.release(mark)
