@@ -48,7 +48,10 @@ struct WsParams {
 //   WS_TAP_*: tap-major order (C a multiple of 16): the 16 rows of a unit are 16 consecutive channels of one
 //             filter tap; tap and first channel follow from the unit number in scalar registers.
 //   WS_TABLE: any order, through the row table (offset from the window origin, r << 16 | s).
-enum { WS_TAP_INSIDE = 0, WS_TAP_MASKED = 1, WS_TABLE = 2 };
+//   WS_ROW3:  tap-major layers with 3 taps per window row: the three taps of a window row are three consecutive
+//             floats of x, so one 12-byte load per (channel, pixel, window row) feeds three units -- a third of the
+//             gather instructions of WS_TAP_MASKED, and instruction issue is what a workgroup runs out of.
+enum { WS_TAP_INSIDE = 0, WS_TAP_MASKED = 1, WS_TABLE = 2, WS_ROW3 = 3 };
 
 template <int MT, int NT, int NW, int MODE>
 __global__ __launch_bounds__(64 * NW) void igemm_wavesplit_kernel(const WsParams p) {
@@ -108,6 +111,33 @@ __global__ __launch_bounds__(64 * NW) void igemm_wavesplit_kernel(const WsParams
         }
         if (MODE != WS_TABLE) pre[nt] += 4u * (uint32_t)g * p.chanStep;      // step j adds j channels
     }
+    // WS_ROW3: the load of a window row starts at its first column inside the image (left padding of at most one
+    // column: the values then sit one component further left); columns outside the image are zeroed after the load,
+    // rows outside poison the whole load.  rowBad: bit r set = window row r outside the image (all set past the last pixel).
+    bool shifted[NT], colBad[NT][3];
+    uint32_t rowBad[NT];
+    if (MODE == WS_ROW3) {
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++) {
+            // bits 0..2 of the tap mask are the columns of window row 0 when that row is inside; rebuilt from the pixel here
+            const long pix = (long)pb * (16 * NT) + nt * 16 + col;
+            shifted[nt] = false;
+            colBad[nt][0] = colBad[nt][1] = colBad[nt][2] = true;
+            rowBad[nt] = ~0u;
+            if (pix < p.Npix) {
+                const uint32_t n = fc_div((uint32_t)pix, p.divOHW);
+                const uint32_t pp = (uint32_t)pix - n * (uint32_t)OHW;
+                const uint32_t oh = fc_div(pp, p.divOW), ow = pp - oh * p.OW;
+                const int ih0 = (int)oh * p.sh - p.pt, iw0 = (int)ow * p.sw - p.pl;
+                shifted[nt] = iw0 < 0;
+#pragma unroll
+                for (int q = 0; q < 3; q++) colBad[nt][q] = !((unsigned)(iw0 + q) < (unsigned)p.W);
+                rowBad[nt] = 0;
+                for (int r = 0; r < p.kh; r++) rowBad[nt] |= ((unsigned)(ih0 + r) < (unsigned)p.H) ? 0u : (1u << r);
+                if (shifted[nt]) pre[nt] += 4u;
+            }
+        }
+    }
     __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.x), 0, p.xBytes, 0x00020000);
 
     __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.Wq), 0, p.wqBytes, 0x00020000);
@@ -164,29 +194,86 @@ __global__ __launch_bounds__(64 * NW) void igemm_wavesplit_kernel(const WsParams
 #pragma unroll
         for (int nt = 0; nt < NT; nt++) acc[mt][nt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    // units of this wavefront: wave, wave + NW, ...
-    const int myUnits = wave < p.nUnits ? (p.nUnits - wave + NW - 1) / NW : 0;
-    const int lastUnit = p.nUnits - 1;
-    auto request = [&](const int i, floatx4 (&a)[MT], float (&b)[NT][4]) __attribute__((always_inline)) {
-        load(min(wave + i * NW, lastUnit), i < myUnits ? 0u : 0x80000000u, a, b);
-    };
-    floatx4 ra[PF][MT];
-    float rb[PF][NT][4];
+    if (MODE == WS_ROW3) {
+        // items of this wavefront: (window row r, block of 16 channels cb) = wave, wave + NW, ...; an item is the three
+        // units (r, 0..2) of that channel block
+        typedef float floatx3 __attribute__((ext_vector_type(3)));
+        const int cpb = p.unitsPerTap, nItems = p.kh * cpb;
+        const int myItems = wave < nItems ? (nItems - wave + NW - 1) / NW : 0;
+        constexpr int PFR = MT * NT >= 4 ? 1 : 2;
+        floatx4 ia[PFR][3][MT];
+        floatx3 ib[PFR][NT][4];
+        auto requestItem = [&](const int i, floatx4 (&a)[3][MT], floatx3 (&b)[NT][4]) __attribute__((always_inline)) {
+            const int it = min(wave + i * NW, nItems - 1);
+            const uint32_t dead = i < myItems ? 0u : 0x80000000u;
+            const uint32_t r = fc_div((uint32_t)it, p.divUnitsPerTap), cb = (uint32_t)it - r * (uint32_t)cpb;
 #pragma unroll
-    for (int i = 0; i < PF; i++) request(i, ra[i], rb[i]);
-    for (int it = 0; it < myUnits; it += PF) {
+            for (int q = 0; q < 3; q++) {
+                const uint32_t aUnit = aTile + ((r * 3u + q) * (uint32_t)cpb + cb) * 1024u;
 #pragma unroll
-        for (int i = 0; i < PF; i++) {
-            if (it + i < myUnits) {
+                for (int mt = 0; mt < MT; mt++)
+                    a[q][mt] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(wres, (aLane + (aUnit + (uint32_t)mt * aBlock)) | dead, 0, 0));
+            }
+            const uint32_t sOff = 4u * r * (uint32_t)p.W + cb * 16u * p.chanStep;
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++) {
+                const uint32_t poison = dead | (((rowBad[nt] >> r) & 1u) << 31);
 #pragma unroll
                 for (int j = 0; j < 4; j++)
-#pragma unroll
-                    for (int mt = 0; mt < MT; mt++)
-#pragma unroll
-                        for (int nt = 0; nt < NT; nt++)
-                            acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[i][mt][j], rb[i][nt][j], acc[mt][nt], 0, 0, 0);
+                    b[nt][j] = __builtin_bit_cast(floatx3, __builtin_amdgcn_raw_buffer_load_b96(
+                                   xres, (pre[nt] + (sOff + (uint32_t)j * p.chanStep)) | poison, 0, 0));
             }
-            request(it + i + PF, ra[i], rb[i]);
+        };
+#pragma unroll
+        for (int i = 0; i < PFR; i++) requestItem(i, ia[i], ib[i]);
+        for (int it = 0; it < myItems; it += PFR) {
+#pragma unroll
+            for (int i = 0; i < PFR; i++) {
+                if (it + i < myItems) {
+#pragma unroll
+                    for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const floatx3 v = ib[i][nt][j];
+                            float t[3];
+                            t[0] = colBad[nt][0] ? 0.f : v[0];
+                            t[1] = colBad[nt][1] ? 0.f : (shifted[nt] ? v[0] : v[1]);
+                            t[2] = colBad[nt][2] ? 0.f : (shifted[nt] ? v[1] : v[2]);
+#pragma unroll
+                            for (int q = 0; q < 3; q++)
+#pragma unroll
+                                for (int mt = 0; mt < MT; mt++)
+                                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(ia[i][q][mt][j], t[q], acc[mt][nt], 0, 0, 0);
+                        }
+                }
+                requestItem(it + i + PFR, ia[i], ib[i]);
+            }
+        }
+    } else {
+        // units of this wavefront: wave, wave + NW, ...
+        const int myUnits = wave < p.nUnits ? (p.nUnits - wave + NW - 1) / NW : 0;
+        const int lastUnit = p.nUnits - 1;
+        auto request = [&](const int i, floatx4 (&a)[MT], float (&b)[NT][4]) __attribute__((always_inline)) {
+            load(min(wave + i * NW, lastUnit), i < myUnits ? 0u : 0x80000000u, a, b);
+        };
+        floatx4 ra[PF][MT];
+        float rb[PF][NT][4];
+    #pragma unroll
+        for (int i = 0; i < PF; i++) request(i, ra[i], rb[i]);
+        for (int it = 0; it < myUnits; it += PF) {
+    #pragma unroll
+            for (int i = 0; i < PF; i++) {
+                if (it + i < myUnits) {
+    #pragma unroll
+                    for (int j = 0; j < 4; j++)
+    #pragma unroll
+                        for (int mt = 0; mt < MT; mt++)
+    #pragma unroll
+                            for (int nt = 0; nt < NT; nt++)
+                                acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[i][mt][j], rb[i][nt][j], acc[mt][nt], 0, 0, 0);
+                }
+                request(it + i + PF, ra[i], rb[i]);
+            }
         }
     }
 
@@ -261,6 +348,7 @@ void ws_launch(fc_context *ctx, const WsParams &p, int mode) {
     const dim3 grid((unsigned)(((p.nKB * p.nPB + 7) / 8) * 8)), block(64 * NW);
     if (mode == WS_TAP_INSIDE) igemm_wavesplit_kernel<MT, NT, NW, WS_TAP_INSIDE><<<grid, block, 0, ctx->stream>>>(p);
     else if (mode == WS_TAP_MASKED) igemm_wavesplit_kernel<MT, NT, NW, WS_TAP_MASKED><<<grid, block, 0, ctx->stream>>>(p);
+    else if (mode == WS_ROW3) igemm_wavesplit_kernel<MT, NT, NW, WS_ROW3><<<grid, block, 0, ctx->stream>>>(p);
     else igemm_wavesplit_kernel<MT, NT, NW, WS_TABLE><<<grid, block, 0, ctx->stream>>>(p);
 }
 
@@ -291,10 +379,10 @@ bool fc_igemm_ws_supports(const fc_conv_shape *s) {
 // split over workgroups; -1 when they should keep the layer.  Read off per-configuration times of the
 // ResNet-50 and VGG-16 layers at batch 1 to 32 and of a dozen other shapes on MI355X.  What a workgroup costs
 // is vector-memory instruction issue (MT + 4*NT loads per unit whatever their width), so the largest tile
-// that still spreads over the chip wins (64x32 from 768 workgroups on, 32x32 and 32x16 from 128, else 16x16),
+// that still spreads over the chip wins (64x32, 32x32 or 32x16 from 192 workgroups on, else 16x16),
 // unless a smaller one pads the layer less.
-// 8 wavefronts over the reduction, 4 when it is shorter than 16 units, 16 when it is long (128 units and
-// more) and the layer has at least 256 pixels.  Beyond about 8 GFLOP (2 GFLOP for strided layers, whose
+// 8 wavefronts over the reduction, 4 when it is shorter than 16 units (16 wavefronts are ahead by 3-5 % on a
+// few long reductions at batch 8 to 16 and behind by 10 % on 256 -> 256 channels at 56x56: not chosen).  Beyond about 8 GFLOP (2 GFLOP for strided layers, whose
 // gathered rows use half of every cache line) the LDS-tiled kernels are level or ahead despite their second launch.
 int fc_igemm_ws_choose(const fc_conv_shape *s, long Npix) {
     if (!fc_igemm_ws_supports(s)) return -1;
@@ -302,7 +390,7 @@ int fc_igemm_ws_choose(const fc_conv_shape *s, long Npix) {
     if (flops > (s->sh > 1 || s->sw > 1 ? 2.0e9 : 8.0e9)) return -1;
     const int nUnits = (s->C * s->kh * s->kw + 15) / 16;
     // among the tiles that bring enough workgroups, the least padded work, weighted by what a product costs in loads
-    static const struct { int mt, nt; long minWgs; double weight; } kTiles[4] = {{4, 2, 768, 1.00}, {2, 2, 128, 1.15}, {2, 1, 128, 1.30}, {1, 1, 0, 1.70}};
+    static const struct { int mt, nt; long minWgs; double weight; } kTiles[4] = {{4, 2, 192, 1.00}, {2, 2, 192, 1.15}, {2, 1, 192, 1.30}, {1, 1, 0, 1.70}};
     int mt = 1, nt = 1;
     double bestCost = 1e300;
     for (int i = 0; i < 4; i++) {
@@ -311,8 +399,7 @@ int fc_igemm_ws_choose(const fc_conv_shape *s, long Npix) {
         const double cost = (double)(kBlocks * 16 * kTiles[i].mt) * (double)(pBlocks * 16 * kTiles[i].nt) * kTiles[i].weight;
         if (cost < bestCost) { bestCost = cost; mt = kTiles[i].mt; nt = kTiles[i].nt; }
     }
-    int nw = nUnits >= 128 && Npix >= 256 ? 16 : nUnits >= 16 ? 8 : 4;
-    if (mt == 4 && nw == 16) nw = 8;      // no 16-wavefront 64x32 configuration: its partial tiles would not fit 64 KB of LDS
+    const int nw = nUnits >= 16 ? 8 : 4;
     for (int i = 0; i < kNumWsShapes; i++)
         if (kWsShapes[i].mt == mt && kWsShapes[i].nt == nt && kWsShapes[i].nw == nw) return i;
     return -1;
@@ -354,7 +441,9 @@ int fc_igemm_ws_run(fc_context *ctx, const fc_igemm_plan *plan, int index, const
     p.pixFastest = (double)plan->Kred_pad * plan->K_pad > (double)s.N * s.C * s.H * s.W ? 1 : 0;
     if ((long)p.nKB * p.nPB >= (1l << 31) - 8) return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_conv_implicit_gemm: grid too large", hipSuccess);
     const bool inside = s.pt == 0 && s.pl == 0 && (plan->OH - 1) * s.sh + s.kh <= s.H && (plan->OW - 1) * s.sw + s.kw <= s.W;
-    const int mode = !tapMajor ? WS_TABLE : inside ? WS_TAP_INSIDE : WS_TAP_MASKED;
+    // three taps per window row and at most one column of left padding: a 12-byte load per window row
+    const bool row3 = tapMajor && s.kw == 3 && s.pl <= 1 && s.kh <= 31;
+    const int mode = !tapMajor ? WS_TABLE : row3 ? WS_ROW3 : inside ? WS_TAP_INSIDE : WS_TAP_MASKED;
     fc_stage_scope scope(ctx, timed ? FC_STAGE_IMPLICIT_GEMM : -1);
 #define FC_WS_CASE(I, MT_, NT_, NW_) case I: ws_launch<MT_, NT_, NW_>(ctx, p, mode); break
     switch (index) {
