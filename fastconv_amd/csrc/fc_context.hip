@@ -101,6 +101,7 @@ extern "C" int fc_destroy(fc_context *ctx) {
     }
     if (ctx->probe_buf) (void)hipFree(ctx->probe_buf);
     (void)hipStreamDestroy(ctx->stream);
+    fc_igemm_static_release(ctx);
     ctx->magic = 0;
     delete ctx;
     return FC_OK;

@@ -56,6 +56,8 @@ static const uint32_t FC_GRAPH_MAGIC = 0x46434752u; // "FCGR"
 int fc_set_error(fc_context *ctx, int status, const char *what, hipError_t err);
 // implicit_gemm.hip: looks up the static workspace of this context's device (once per device)
 int fc_igemm_static_init(fc_context *ctx);
+// gives the static workspace of the context's device back when this context was the one using it
+void fc_igemm_static_release(fc_context *ctx);
 bool fc_ctx_ok(const fc_context *ctx);
 // implicit_gemm_wavesplit.hip: the implicit-GEMM configurations whose workgroups split the reduction over their
 // wavefronts (small tiles, one launch per layer, for layers with few output pixels).  `index` counts them from 0;

@@ -704,7 +704,17 @@ static __device__ __align__(256) float scratch[FC_IGEMM_STATIC_WS_BYTES / sizeof
 static const int kMaxDevices = 64;
 static float *g_scratch_ptr[kMaxDevices];
 static bool g_scratch_known[kMaxDevices];
+// The context that uses the array of a device: the first one to call fc_conv_implicit_gemm_static there, until it is
+// destroyed.  Calls of one context are ordered on its stream; another context's would race with them, so they are refused.
+static fc_context *g_scratch_owner[kMaxDevices];
 static std::mutex g_scratch_mutex;
+
+// Called by fc_destroy.
+void fc_igemm_static_release(fc_context *ctx) {
+    if (ctx->device < 0 || ctx->device >= kMaxDevices) return;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_owner[ctx->device] == ctx) g_scratch_owner[ctx->device] = nullptr;
+}
 
 // Called by fc_init with ctx->device current.
 int fc_igemm_static_init(fc_context *ctx) {
@@ -735,6 +745,14 @@ extern "C" int fc_conv_implicit_gemm_static(fc_context *ctx, const fc_igemm_plan
         return fc_set_error(ctx, FC_ERR_UNSUPPORTED, msg, hipSuccess);
     }
     if (!ctx->igemm_static_ws) return fc_set_error(ctx, FC_ERR_STATE, "fc_conv_implicit_gemm_static: static workspace not set up", hipSuccess);
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        fc_context *&owner = g_scratch_owner[ctx->device];
+        if (owner == nullptr) owner = ctx;
+        if (owner != ctx)
+            return fc_set_error(ctx, FC_ERR_STATE, "fc_conv_implicit_gemm_static: the static workspace of this GPU is in use by another "
+                                "context (one context per GPU may use it at a time; it is free again once that context is destroyed)", hipSuccess);
+    }
     // Nothing has to start at zero: every partial sum the reduction reads ([split][k < K][pixel < Npix]) is
     // written by this call's GEMM kernel first.  No event brackets (creating an event may allocate).
     return igemm_run(ctx, plan, x_dev, Wp_dev, table_dev, bias_dev, relu, ctx->igemm_static_ws, y_dev, false,

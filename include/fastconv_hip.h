@@ -370,8 +370,11 @@ int fc_conv_implicit_gemm(fc_context *ctx, const fc_igemm_plan *plan, const floa
  * inside the library instead of a workspace of the caller's (each GPU the library runs on holds
  * that array until the process ends); the call allocates nothing and is never bracketed by
  * timing events.  A plan whose ws_bytes exceeds FC_IGEMM_STATIC_WS_BYTES is refused with
- * FC_ERR_UNSUPPORTED.  All calls on one GPU share the array: calls that overlap in time on
- * one GPU (two contexts, two streams) race; calls on one context are ordered and safe. */
+ * FC_ERR_UNSUPPORTED.  All calls on one GPU share the array and calls that overlapped in time
+ * would race, so one context per GPU uses it at a time: the first context to make this call on a
+ * GPU owns the array until fc_destroy, and the call is refused for any other context meanwhile
+ * (FC_ERR_STATE); calls of one context are ordered on its stream and safe.  Other processes have
+ * their own copy of the array. */
 #define FC_IGEMM_STATIC_WS_BYTES (32 << 20)
 int fc_conv_implicit_gemm_static(fc_context *ctx, const fc_igemm_plan *plan, const float *x_dev,
                                  const float *Wp_dev, const int32_t *table_dev,

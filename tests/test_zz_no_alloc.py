@@ -87,8 +87,27 @@ def test_static_workspace_entry_point_matches_the_caller_workspace_one():
         with pytest.raises(F.FastConvError) as e:
             L.conv_implicit_gemm_static(ok, None, buf, buf, buf)
         assert "fc_conv_implicit_gemm_static:" in str(e.value)
+        # a second context on the same GPU is refused while this one owns the array, and served once it is gone
+        other = F.load(0, 64 << 20)
+        try:
+            obuf = other.alloc(1 << 20)
+            with pytest.raises(F.FastConvError) as e:
+                other.conv_implicit_gemm_static(ok, obuf, obuf, obuf, obuf)
+            assert e.value.status == -5 and "another context" in str(e.value)
+            L.close()
+            L = None
+            ow, ox = other.alloc(1 << 20), other.alloc(1 << 20)
+            other.fill_zero(ow, 1 << 20)
+            other.fill_zero(ox, 1 << 20)
+            oWp, otab, oy = other.alloc(ok.Wp_bytes), other.alloc(ok.table_bytes), other.alloc(1 << 20)
+            other.igemm_pack_filter(ok, ow, oWp, otab)
+            other.conv_implicit_gemm_static(ok, ox, oWp, otab, oy)
+            assert not other.download(oy, (1, 16, 8, 8)).any()
+        finally:
+            other.close()
     finally:
-        L.close()
+        if L is not None:
+            L.close()
 
 
 def test_static_workspace_entry_point_inside_a_recorded_graph():
