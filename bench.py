@@ -340,6 +340,9 @@ def run_workload(name, steps, warmup, o, detail=True, offline_filter=None):
     """Builds the layers of one workload on the device, times `steps` steps and returns the result fields."""
     import fastconv_amd as F
     layers_def, N, algo, desc = WORKLOADS[name]
+    if getattr(o, "batch", 0):
+        N = o.batch
+        desc += " (batch overridden: %d)" % N
     stress = name.startswith("stress")
     tune = o.tune or stress
 
@@ -804,6 +807,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="vgg16_b32", choices=sorted(WORKLOADS))
+    ap.add_argument("--batch", type=int, default=0, metavar="N",
+                    help="run the workload's layers at batch N instead of its own batch (the crossover of the two "
+                         "algorithms between batch 1 and 32 is measured this way)")
     ap.add_argument("--tune", action="store_true",
                     help="search tile shape, pipeline and algorithm per layer before timing (default: the library's "
                          "untuned choices; the stress workloads always search)")

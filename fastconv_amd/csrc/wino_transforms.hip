@@ -455,19 +455,19 @@ extern "C" int fc_wino_make_plan(const fc_conv_shape *s, int gemm_config, fc_win
 }
 
 // Measured on MI355X (both algorithms at their best tile shape, whole-layer forward time, every 3x3
-// stride-1 layer of VGG-16 and ResNet-50 at batch 1 and 32): Winograd wins on every layer with at
-// least 1.85 GFLOP of direct-convolution work and 16 or more input channels (by 1.25x to 3.9x); on the
-// batch-1 layers of 0.92 GFLOP or less one implicit-GEMM launch is level with the three launches of
-// the staged pipeline (within 4 % on three of five layers, 1.2-1.4x ahead on two) and is what the rule
-// takes; on the 3-channel first layer the two are level at batch 32 (both bound by the stores of the
-// output) and the implicit GEMM is 2.1x ahead at batch 1.
+// stride-1 layer of VGG-16 and ResNet-50 at batch 1, 4 and 32, the ResNet-50 ones also at 8 and 16): with
+// 16 or more input channels Winograd wins from 3.7 GFLOP of direct-convolution work on (by 1.1x to 3.2x;
+// two 512-channel layers are level there); at 1.85 GFLOP the two are level (seven layers, 0.97-1.36);
+// up to 0.92 GFLOP one implicit-GEMM launch, its reduction split inside the workgroups, is 1.3-2.2x ahead
+// of the three launches of the staged pipeline.  The 3-channel first layer: implicit GEMM 1.5-1.7x ahead
+// at batch 1 and 4, the two within 10 % at batch 32 (both bound by the stores of the output).
 extern "C" int fc_prefer_winograd(const fc_conv_shape *s) {
     if (!fc_shape_ok(s) || s->kh != 3 || s->kw != 3 || s->sh != 1 || s->sw != 1) return 0;
     const int OH = fc_out_dim(s->H, s->pt, s->pb, 3, 1), OW = fc_out_dim(s->W, s->pl, s->pr, 3, 1);
     if ((OW + 5) / 6 > kWinoMaxTilesW) return 0;
     if (s->C < 16) return 0;
     const double flop = 2.0 * s->N * s->K * s->C * (double)OH * OW * 9.0;
-    return flop >= 1.3e9 ? 1 : 0;
+    return flop >= 2.5e9 ? 1 : 0;
 }
 
 static int plan_check(fc_context *ctx, const fc_wino_plan *plan, const void *a, const void *b) {

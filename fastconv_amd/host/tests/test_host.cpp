@@ -108,20 +108,28 @@ static void test_select_algorithm() {
     CHECK(select_algorithm(k3, s2, o56, 256, 256, 32) == nnp_convolution_algorithm_im2col);
     CHECK(select_algorithm(k1, s2, o56, 256, 512, 1) == nnp_convolution_algorithm_im2col);
     CHECK(select_algorithm(k7, s2, o224, 3, 64, 1) == nnp_convolution_algorithm_im2col);
-    // 3x3 stride 1: the rule must pick the measured winner on every VGG-16 / ResNet-50 layer at batch 1
-    // and 32 (whole-layer milliseconds on MI355X, Winograd and implicit GEMM at their best tile shape);
+    // 3x3 stride 1: the rule must pick the measured winner on every VGG-16 / ResNet-50 layer at batch 1, 4
+    // and 32 and on the ResNet-50 layers at batch 8 and 16, where the two algorithms cross (whole-layer
+    // milliseconds on MI355X, Winograd and implicit GEMM at their best tile shape);
     // layers where the two are within 15 % of each other may go either way (boxes of the pool differ by up to that
     // much on layers bound by their stores, such as the 3-channel first layer)
     static const struct { int c, k, h, n; double wino_ms, im2col_ms; } measured[] = {
-        {3, 64, 224, 1, 0.0256, 0.0119}, {64, 64, 224, 1, 0.0370, 0.0510}, {64, 128, 112, 1, 0.0300, 0.0376},
-        {128, 128, 112, 1, 0.0326, 0.0567}, {128, 256, 56, 1, 0.0305, 0.0383}, {256, 256, 56, 1, 0.0342, 0.0533},
-        {256, 512, 28, 1, 0.0270, 0.0349}, {512, 512, 28, 1, 0.0344, 0.0511}, {512, 512, 14, 1, 0.0302, 0.0311},
-        {64, 64, 56, 1, 0.0196, 0.0168}, {128, 128, 28, 1, 0.0193, 0.0201}, {256, 256, 14, 1, 0.0216, 0.0220},
-        {512, 512, 7, 1, 0.0306, 0.0214}, {3, 64, 224, 32, 0.1222, 0.1308}, {64, 64, 224, 32, 0.4934, 1.0072},
-        {64, 128, 112, 32, 0.2665, 0.4752}, {128, 128, 112, 32, 0.4265, 0.9336}, {128, 256, 56, 32, 0.1987, 0.4774},
-        {256, 256, 56, 32, 0.3187, 0.9552}, {256, 512, 28, 32, 0.1654, 0.4999}, {512, 512, 28, 32, 0.2967, 1.0109},
-        {512, 512, 14, 32, 0.1338, 0.2825}, {64, 64, 56, 32, 0.0546, 0.0779}, {128, 128, 28, 32, 0.0462, 0.0881},
-        {256, 256, 14, 32, 0.0532, 0.0854}, {512, 512, 7, 32, 0.0726, 0.0852}};
+        {3, 64, 224, 1, 0.0203, 0.0117}, {64, 64, 224, 1, 0.0367, 0.0486}, {64, 128, 112, 1, 0.0301, 0.0302},
+        {128, 128, 112, 1, 0.0330, 0.0491}, {128, 256, 56, 1, 0.0304, 0.0284}, {256, 256, 56, 1, 0.0341, 0.0469},
+        {256, 512, 28, 1, 0.0268, 0.0277}, {512, 512, 28, 1, 0.0341, 0.0463}, {512, 512, 14, 1, 0.0302, 0.0190},
+        {64, 64, 56, 1, 0.0198, 0.0107}, {128, 128, 28, 1, 0.0193, 0.0105}, {256, 256, 14, 1, 0.0214, 0.0107},
+        {512, 512, 7, 1, 0.0307, 0.0141}, {3, 64, 224, 4, 0.0332, 0.0217}, {64, 64, 224, 4, 0.0922, 0.1397},
+        {64, 128, 112, 4, 0.0465, 0.0802}, {128, 128, 112, 4, 0.0628, 0.1381}, {128, 256, 56, 4, 0.0418, 0.0798},
+        {256, 256, 56, 4, 0.0587, 0.1428}, {256, 512, 28, 4, 0.0447, 0.0809}, {512, 512, 28, 4, 0.0683, 0.1505},
+        {512, 512, 14, 4, 0.0474, 0.0468}, {64, 64, 56, 4, 0.0256, 0.0194}, {128, 128, 28, 4, 0.0253, 0.0185},
+        {256, 256, 14, 4, 0.0290, 0.0192}, {512, 512, 7, 4, 0.0313, 0.0190}, {64, 64, 56, 8, 0.0322, 0.0309},
+        {128, 128, 28, 8, 0.0306, 0.0284}, {256, 256, 14, 8, 0.0372, 0.0274}, {512, 512, 7, 8, 0.0361, 0.0296},
+        {64, 64, 56, 16, 0.0368, 0.0474}, {128, 128, 28, 16, 0.0360, 0.0478}, {256, 256, 14, 16, 0.0415, 0.0464},
+        {512, 512, 7, 16, 0.0519, 0.0467}, {3, 64, 224, 32, 0.1206, 0.1312}, {64, 64, 224, 32, 0.4979, 1.0260},
+        {64, 128, 112, 32, 0.2675, 0.4769}, {128, 128, 112, 32, 0.4275, 0.9476}, {128, 256, 56, 32, 0.1979, 0.4817},
+        {256, 256, 56, 32, 0.3231, 0.9416}, {256, 512, 28, 32, 0.1670, 0.4903}, {512, 512, 28, 32, 0.2932, 0.9387},
+        {512, 512, 14, 32, 0.1314, 0.2724}, {64, 64, 56, 32, 0.0538, 0.0797}, {128, 128, 28, 32, 0.0459, 0.0781},
+        {256, 256, 14, 32, 0.0533, 0.0798}, {512, 512, 7, 32, 0.0741, 0.0835}};
     for (size_t i = 0; i < sizeof measured / sizeof measured[0]; i++) {
         const nnp_size o = {(size_t)measured[i].h, (size_t)measured[i].h};
         const bool wino = select_algorithm(k3, s1, o, measured[i].c, measured[i].k, measured[i].n) == nnp_convolution_algorithm_winograd;
