@@ -79,6 +79,8 @@ WORKLOADS = {
     "igemm_3x3s2_b32": ([(128, 128, 56, 3, 2, 1, 1)], 32, "im2col", "single 3x3 stride-2 conv 128->128 @56, implicit GEMM, batch 32 (ResNet-50 conv3 entry)"),
     "igemm_1x1_b32": ([(256, 64, 56, 1, 1, 0, 1)], 32, "im2col", "single 1x1 conv 256->64 @56, implicit GEMM, batch 32 (ResNet-50 bottleneck reduce)"),
     "igemm_stem_b32": ([(3, 64, 224, 7, 2, 3, 1)], 32, "im2col", "single 7x7 stride-2 conv 3->64 @224, implicit GEMM, batch 32 (ResNet-50 stem)"),
+    "igemm_512_7_b1": ([(512, 512, 7, 3, 1, 1, 1)], 1, "im2col", "single 3x3 conv 512->512 @7, implicit GEMM, batch 1 (ResNet-50 conv5): 49 pixels, reduction split over wavefronts"),
+    "igemm_2048_512_7_b1": ([(2048, 512, 7, 1, 1, 0, 1)], 1, "im2col", "single 1x1 conv 2048->512 @7, implicit GEMM, batch 1 (ResNet-50 conv5 reduce): 49 pixels"),
     "stress_b64": (_w(STRESS), 64, "winograd", "VGG-16 256@56, 512@28, 512@14 at batch 64: staged (ZC) against blocked Winograd, tile shapes searched"),
     "stress_b128": (_w(STRESS), 128, "winograd", "VGG-16 256@56, 512@28, 512@14 at batch 128: staged (ZC) against blocked Winograd, tile shapes searched"),
 }
