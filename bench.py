@@ -85,7 +85,8 @@ WORKLOADS = {
     "stress_b128": (_w(STRESS), 128, "winograd", "VGG-16 256@56, 512@28, 512@14 at batch 128: staged (ZC) against blocked Winograd, tile shapes searched"),
 }
 # (workload, filter transform offline): compact results a default run appends
-SECONDARY = (("vgg16_b1", False), ("vgg16_b1", True), ("resnet50_b32", False), ("resnet50_b1", False), ("im2col_abc_b1", False))
+SECONDARY = (("vgg16_b1", False), ("vgg16_b1", True), ("vgg16_auto_b1", False), ("resnet50_b32", False), ("resnet50_b1", False),
+             ("im2col_abc_b1", False))
 
 ST_KT, ST_IT, ST_GEMM, ST_OT, ST_IGEMM, ST_FUSED, ST_ONEPASS = 0, 1, 2, 3, 4, 6, 7
 
@@ -850,6 +851,7 @@ def main():
 
     out = run_workload(args.workload, args.steps, args.warmup, args)
     if args.workload == "vgg16_b32" and not (args.no_secondary or args.timed_only):
+        args.batch = 0      # the secondary workloads run at their own batch
         out["secondary"] = [compact(run_workload(w, min(args.steps, 20), args.warmup, args, detail=False,
                                                  offline_filter=off)) for (w, off) in SECONDARY]
     if not args.no_cpu_baseline:
