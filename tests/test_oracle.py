@@ -102,7 +102,7 @@ def test_all_ones_closed_form(shape):
         assert np.array_equal(y, np.broadcast_to(expect, y.shape))
     if s.kh == 3 and s.kw == 3 and s.sh == 1:
         assert np.allclose(O.wino_conv_f32(s, x, w), expect, rtol=0, atol=1e-4)
-    # the two values the reference survey quotes for 8ch 9x9 s2 p1: corner 32, centre 72
+    # by hand for 8 channels, 9x9, stride 2, padding 1: a corner output sees 2x2 taps (32), a centre one 3x3 (72)
     if shape[1] == 8:
         assert expect[0, 0] == 32 and expect[2, 2] == 72
 
