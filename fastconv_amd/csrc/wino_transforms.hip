@@ -305,9 +305,12 @@ struct OutTParams {
 
 // Block = one output channel x TPB consecutive tiles, one thread per tile.  The 64
 // plane loads of a wavefront are each 256 contiguous bytes.  The 6x6 results are
-// laid into LDS as the image rows they cover ([band][6][OW]) and copied out band
-// by band: a band the block covers completely is one contiguous run of rows*OW
-// floats, a partly covered band (first or last of the range) is one run per row.
+// laid into LDS as the image rows they cover, row after row exactly as in y (a
+// band of a 14-row image whose tiles reach past the last row takes 2 rows, not 6),
+// and copied out image by image: the bands of an image that the block covers
+// completely are one contiguous run of rows*OW floats in LDS and in y (a whole
+// 14x14 image leaves in one 16-byte store per lane instead of five 4-byte ones),
+// a partly covered band (first or last of the range) is one run per row.
 // Everything that does not depend on the lane (plane bases, band geometry of the
 // copy loop) is kept in scalar registers: the kernel spends a quarter of its
 // vector instructions on addresses otherwise.
@@ -316,7 +319,7 @@ struct OutTParams {
 // per byte for 128 more registers.
 template <int TPB, int TPT = 1>
 __global__ __launch_bounds__(TPB / TPT) void wino_output_transform_kernel(const OutTParams p) {
-    extern __shared__ __attribute__((aligned(16))) float lds[];   // [bands][6][OW]
+    extern __shared__ __attribute__((aligned(16))) float lds[];   // image rows of OW floats, at most 6 per band
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int k = blockIdx.y;
@@ -325,8 +328,9 @@ __global__ __launch_bounds__(TPB / TPT) void wino_output_transform_kernel(const 
     const uint32_t tLast = min((uint32_t)(t0 + TPB), (uint32_t)p.T) - 1;
     const uint32_t gb0 = fc_div(t0, p.divTW), gbL = fc_div(tLast, p.divTW);
     const int tw0 = t0 - gb0 * p.tW, twL = tLast - gbL * p.tW;
-    const int NB = (int)(gbL - gb0) + 1;
-    const int bandElems = 6 * p.OW;
+    // image rows in LDS: row (n*OH + th*6 + i) - row0 for band n*tH + th, row0 = first row of the first band
+    const uint32_t n0 = fc_div(gb0, p.divTH), nL = fc_div(gbL, p.divTH);
+    const int row0 = (int)n0 * p.OH + (int)(gb0 - n0 * p.tH) * 6;
 
     const uint32_t tFirst = t0 + TPT * tid;
     if (tFirst <= tLast) {
@@ -355,7 +359,9 @@ __global__ __launch_bounds__(TPB / TPT) void wino_output_transform_kernel(const 
             const uint32_t t = tFirst + u;
             if (t > tLast) break;
             const uint32_t gb = fc_div(t, p.divTW);
-            const int q = t - gb * p.tW, j = gb - gb0;
+            const int q = t - gb * p.tW;
+            const uint32_t n = fc_div(gb, p.divTH);
+            const int th = (int)(gb - n * p.tH);
             float tmp[6][8];
 #pragma unroll
             for (int jj = 0; jj < 8; jj++) {
@@ -365,8 +371,9 @@ __global__ __launch_bounds__(TPB / TPT) void wino_output_transform_kernel(const 
 #pragma unroll
                 for (int i = 0; i < 6; i++) tmp[i][jj] = s[i];
             }
-            float *img = lds + j * bandElems + q * 6;
+            float *img = lds + ((int)n * p.OH + th * 6 - row0) * p.OW + q * 6;
             const int colsLeft = p.OW - q * 6;      // columns of this tile inside the image
+            const int rowsLeft = p.OH - th * 6;     // and rows: the rows below belong to the next image in LDS
 #pragma unroll
             for (int i = 0; i < 6; i++) {
                 // the bias goes in with element 1: at6 adds it (as m1 + m2 or m1 - m2) to each of its six outputs once
@@ -376,13 +383,15 @@ __global__ __launch_bounds__(TPB / TPT) void wino_output_transform_kernel(const 
 #pragma unroll
                 for (int jj = 0; jj < 6; jj++) s[jj] = __builtin_elementwise_maximum(s[jj], floorv);
                 float *dstl = img + i * p.OW;
-                if (colsLeft >= 6) {
+                if (i < rowsLeft) {
+                    if (colsLeft >= 6) {
 #pragma unroll
-                    for (int jj = 0; jj < 6; jj++) dstl[jj] = s[jj];
-                } else {
+                        for (int jj = 0; jj < 6; jj++) dstl[jj] = s[jj];
+                    } else {
 #pragma unroll
-                    for (int jj = 0; jj < 6; jj++)
-                        if (jj < colsLeft) dstl[jj] = s[jj];
+                        for (int jj = 0; jj < 6; jj++)
+                            if (jj < colsLeft) dstl[jj] = s[jj];
+                    }
                 }
             }
         }
@@ -390,29 +399,43 @@ __global__ __launch_bounds__(TPB / TPT) void wino_output_transform_kernel(const 
     __syncthreads();
 
     constexpr int WAVES = TPB / TPT / 64;
-    const bool vec4 = (p.OW & 3) == 0;
     const size_t chan = (size_t)p.OH * p.OW;
-    for (int j = wave; j < NB; j += WAVES) {       // j and everything derived from it is uniform
-        const uint32_t gb = gb0 + j;
-        const uint32_t n = fc_div(gb, p.divTH), th = gb - n * p.tH;
-        const int rows = min(6, p.OH - (int)th * 6);
-        const int xA = (j == 0) ? tw0 * 6 : 0;
-        const int xB = min((j == NB - 1) ? (twL + 1) * 6 : p.tW * 6, p.OW);
-        float *dst = p.y + ((size_t)n * p.K + k) * chan + (size_t)th * 6 * p.OW;
-        const float *src = lds + j * bandElems;
-        if (xA == 0 && xB == p.OW) {
-            const int len = rows * p.OW;
+    // one row of a partly covered band: columns xA .. xB-1 of `rows` rows
+    auto copy_rows = [&](float *dst, const float *src, int rows, int xA, int xB) {
+        for (int i = 0; i < rows; i++)
+            for (int x = xA + lane; x < xB; x += 64) store_at(dst + i * p.OW, (uint32_t)x * 4u, src[i * p.OW + x]);
+    };
+    for (uint32_t n = n0 + wave; n <= nL; n += WAVES) {       // n and everything derived from it is uniform
+        // bands of image n inside the block, as rows of tiles of that image
+        const uint32_t gbA = max(gb0, n * p.tH), gbB = min(gbL, n * p.tH + p.tH - 1);
+        const int thA = (int)(gbA - n * p.tH), thB = (int)(gbB - n * p.tH);
+        // the first band of the block starts at tile tw0, its last band ends with tile twL
+        const bool cutA = gbA == gb0 && tw0 > 0, cutB = gbB == gbL && (twL + 1) * 6 < p.OW;
+        const bool cutBoth = cutA && cutB && gbA == gbB;      // one band, open on both sides: one copy does it
+        float *img = p.y + ((size_t)n * p.K + k) * chan;
+        const int simg = ((int)n * p.OH - row0) * p.OW;      // where row 0 of the image would lie in LDS
+        if (cutA) {
+            const int xB = (gbA == gbL) ? min((twL + 1) * 6, p.OW) : p.OW;
+            copy_rows(img + thA * 6 * p.OW, lds + (simg + thA * 6 * p.OW), min(6, p.OH - thA * 6), tw0 * 6, xB);
+        }
+        if (cutB && !cutBoth) copy_rows(img + thB * 6 * p.OW, lds + (simg + thB * 6 * p.OW), min(6, p.OH - thB * 6), 0, (twL + 1) * 6);
+        const int cA = thA + (cutA ? 1 : 0), cB = thB - (cutB ? 1 : 0);      // the bands covered completely
+        if (cA <= cB) {
+            const int rowA = cA * 6, rowB = min(p.OH, (cB + 1) * 6);
+            const int len = (rowB - rowA) * p.OW;
+            float *dst = img + rowA * p.OW;
+            const float *src = lds + (simg + rowA * p.OW);
+            // 16-byte pieces where the run starts on a 16-byte boundary in y and in LDS and is a whole number of them
+            const bool vec4 = (len & 3) == 0 && ((((size_t)n * p.K + k) * chan + (size_t)rowA * p.OW) & 3) == 0 &&
+                              ((simg + rowA * p.OW) & 3) == 0;
             if (vec4) {
-                typedef float vec4 __attribute__((ext_vector_type(4)));
+                typedef float vec4f __attribute__((ext_vector_type(4)));
                 for (int e = lane; e < len / 4; e += 64)
-                    *reinterpret_cast<vec4 *>(reinterpret_cast<char *>(dst) + (uint32_t)e * 16u) =
-                        *reinterpret_cast<const vec4 *>(reinterpret_cast<const char *>(src) + (uint32_t)e * 16u);
+                    *reinterpret_cast<vec4f *>(reinterpret_cast<char *>(dst) + (uint32_t)e * 16u) =
+                        *reinterpret_cast<const vec4f *>(reinterpret_cast<const char *>(src) + (uint32_t)e * 16u);
             } else {
                 for (int e = lane; e < len; e += 64) store_at(dst, (uint32_t)e * 4u, src[e]);
             }
-        } else {
-            for (int i = 0; i < rows; i++)
-                for (int x = xA + lane; x < xB; x += 64) store_at(dst + i * p.OW, (uint32_t)x * 4u, src[i * p.OW + x]);
         }
     }
 }
