@@ -455,7 +455,7 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
 #pragma unroll
                         for (int j = 0; j < 4; j++) {
                             float v = acc[mi][ni][q * 4 + j] + bq[j];
-                            if (p.relu) v = fmaxf(v, 0.f);
+                            if (p.relu) v = __builtin_elementwise_maximum(v, 0.f);      // keeps a NaN
                             *reinterpret_cast<float *>(dst + (off + (uint32_t)(mi * 32 + 8 * q + j) * rowStride)) = v;
                         }
                     }
@@ -495,7 +495,7 @@ __global__ __launch_bounds__(TL::THREADS, TL::MIN_WAVES) void igemm_conv_kernel(
                 if (k < p.K) {
                     float v = acc[mi][ni][i];
                     if (p.bias) v += p.bias[k];
-                    if (p.relu) v = fmaxf(v, 0.f);
+                    if (p.relu) v = __builtin_elementwise_maximum(v, 0.f);      // keeps a NaN
                     yn[(size_t)k * OHW] = v;
                 }
             }
@@ -515,7 +515,7 @@ __global__ __launch_bounds__(256) void igemm_reduce_kernel(const float *__restri
     float v = src[0];
     for (int z = 1; z < splitK; z++) v += src[(size_t)z * slab];
     if (bias) v += bias[k];
-    if (relu) v = fmaxf(v, 0.f);
+    if (relu) v = __builtin_elementwise_maximum(v, 0.f);      // keeps a NaN
     const uint32_t n = fc_div((uint32_t)pix, divOHW);
     y[((size_t)n * K + k) * OHW + (pix - (long)n * OHW)] = v;
 }

@@ -295,7 +295,7 @@ __global__ __launch_bounds__(64 * NW) void igemm_wavesplit_kernel(const WsParams
         const long pix = (long)pb * (16 * NT) + nt * 16 + (ln & 15);
         if (k < p.K && pix < p.Npix) {
             if (p.bias) v += p.bias[k];
-            if (p.relu) v = fmaxf(v, 0.f);
+            if (p.relu) v = __builtin_elementwise_maximum(v, 0.f);      // keeps a NaN
             const uint32_t n = fc_div((uint32_t)pix, p.divOHW);
             p.y[((size_t)n * p.K + k) * OHW + ((uint32_t)pix - n * (uint32_t)OHW)] = v;
         }

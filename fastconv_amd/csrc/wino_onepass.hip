@@ -263,7 +263,7 @@ __global__ __launch_bounds__(kFusedThreads, 1) void wino_onepass_kernel(const On
 #pragma unroll
                     for (int jj = 0; jj < 6; jj++) {
                         sres[jj] += bias;
-                        if (p.out.relu) sres[jj] = fmaxf(sres[jj], 0.f);
+                        if (p.out.relu) sres[jj] = __builtin_elementwise_maximum(sres[jj], 0.f);      // keeps a NaN, as the other epilogues do
                     }
                     float *drow = dst + (size_t)i * p.out.OW;
                     if (pairs) {

@@ -254,8 +254,10 @@ def test_winograd_bias_relu_epilogue(lib):
 
 def test_nan_and_inf_reach_the_output_of_every_path(lib):
     """A NaN in the input must come out as NaN (not as -inf or 0) wherever it contributes, with ReLU
-    off, through the staged, fused, single-kernel and small-channel Winograd epilogues and the
-    implicit GEMM; outputs it does not reach stay finite in the implicit GEMM."""
+    off and on (numpy's maximum, which the other tests compare the fused ReLU with, propagates it),
+    through the staged, fused, single-kernel and small-channel Winograd epilogues and the implicit
+    GEMM (LDS-tiled, with a split reduction, and split over the wavefronts); outputs it does not
+    reach stay finite in the implicit GEMM."""
     for shp in [(1, 8, 14, 14, 12), (1, 3, 20, 20, 9)]:
         s = O.shape(*shp)
         cs = cshape(s)
@@ -263,15 +265,19 @@ def test_nan_and_inf_reach_the_output_of_every_path(lib):
         x[0, 1, 5, 6] = np.nan
         bias = O.rng_uniform(2, (s.K,))
         announce("NaN propagation", shp)
+        ws = [c.id for c in lib.igemm_configs() if c.waves_k > 1][0]
         for name, fn in (("staged", lib.winograd_conv), ("fused", lib.winograd_conv_fused),
-                         ("single kernel", lib.winograd_conv_onepass), ("implicit gemm", lib.implicit_gemm_conv)):
-            y = fn(cs, x, w, bias=bias)
-            assert np.isnan(y[0, :, 4:7, 5:8]).all(), name          # the 3x3 windows that hold the NaN
-            assert not np.isinf(y).any(), name
-            if name == "implicit gemm":
-                ok = np.ones(y.shape, bool)
-                ok[0, :, 4:7, 5:8] = False
-                assert np.isfinite(y[ok]).all()
+                         ("single kernel", lib.winograd_conv_onepass), ("implicit gemm", lib.implicit_gemm_conv),
+                         ("implicit gemm, LDS-tiled", lambda *a, **k: lib.implicit_gemm_conv(*a, config=3, **k)),
+                         ("implicit gemm, wavefront split", lambda *a, **k: lib.implicit_gemm_conv(*a, config=ws, **k))):
+            for relu in (False, True):
+                y = fn(cs, x, w, bias=bias, relu=relu)
+                assert np.isnan(y[0, :, 4:7, 5:8]).all(), (name, relu)          # the 3x3 windows that hold the NaN
+                assert not np.isinf(y).any(), (name, relu)
+                if name.startswith("implicit gemm"):
+                    ok = np.ones(y.shape, bool)
+                    ok[0, :, 4:7, 5:8] = False
+                    assert np.isfinite(y[ok]).all()
 
 
 @pytest.mark.parametrize("shp", [
