@@ -641,6 +641,17 @@ def run_workload(name, steps, warmup, o, detail=True, offline_filter=None):
             transforms["copy_kernel"] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                          "frac": round(gbs / PEAK_HBM_GBS, 4), "bytes": 2 * nb,
                                          "note": "read + write of a plain copy: what streaming kernels reach on this box"}
+            # and stores alone (the library's fill kernel): the input transform writes 1.8x what it reads
+            L.fill_zero(M, nb)
+            L.sync()
+            t0c = time.perf_counter()
+            for _ in range(5):
+                L.fill_zero(M, nb)
+            L.sync()
+            gbs = nb * 5 / (time.perf_counter() - t0c) / 1e9
+            transforms["fill_kernel"] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                         "frac": round(gbs / PEAK_HBM_GBS, 4), "bytes": nb,
+                                         "note": "stores only: what a write-bound kernel reaches on this box"}
 
     def class_detail(lay, cand):
         """Time and GEMM-stage MFMA rate of one layer class's best candidate (events around every kernel)."""

@@ -294,6 +294,11 @@ __global__ void fc_fill_zero_kernel(uint32_t *dst, size_t words) {
     for (; i < words; i += stride) dst[i] = 0u;
 }
 
+__global__ __launch_bounds__(256) void fc_fill_zero16_kernel(uint4 *dst, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[i] = make_uint4(0u, 0u, 0u, 0u);
+}
+
 // A fill kernel rather than a memset node, so that callers may record it into a
 // HIP graph.
 extern "C" int fc_fill_zero(fc_context *ctx, void *dst_dev, size_t bytes) {
@@ -301,6 +306,13 @@ extern "C" int fc_fill_zero(fc_context *ctx, void *dst_dev, size_t bytes) {
     if (!dst_dev || (bytes & 3) || ((uintptr_t)dst_dev & 3))
         return fc_set_error(ctx, FC_ERR_INVALID, "fc_fill_zero: pointer and size must be 4-byte multiples", hipSuccess);
     if (bytes == 0) return FC_OK;
+    if (((uintptr_t)dst_dev & 15) == 0 && (bytes & 15) == 0 && bytes / 16 / 256 < (1ull << 31)) {
+        // 16 bytes per lane, one store per thread, as the copy kernel
+        const size_t n = bytes / 16;
+        fc_fill_zero16_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx->stream>>>((uint4 *)dst_dev, n);
+        FC_LAUNCH_CHECK(ctx, "fc_fill_zero16_kernel");
+        return FC_OK;
+    }
     const size_t words = bytes / 4;
     size_t blocks = (words + 255) / 256;
     if (blocks > 4096) blocks = 4096;

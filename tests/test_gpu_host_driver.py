@@ -191,3 +191,26 @@ def test_maxpool_against_numpy():
             assert np.array_equal(y, xe.max(axis=(3, 5)))
     finally:
         L.close()
+
+
+def test_fill_zero_clears_exactly_its_range():
+    """fc_fill_zero with 16-byte-aligned ranges (one 16-byte store per lane) and with ranges aligned
+    to 4 bytes only (4-byte stores): the range reads back as zeros and its neighbours are untouched."""
+    import ctypes
+    import fastconv_amd as F
+    L = F.load(0, 1 << 30)
+    try:
+        n = 1 << 16
+        ones = np.ones(n, np.float32)
+        buf = L.upload(ones)
+        for (first, count) in [(0, n), (4, 4096), (16, 20), (1, 7), (3, 4097), (5, 1), (n - 4, 4), (n - 3, 3)]:
+            L.upload_into(buf, ones)
+            L.fill_zero(ctypes.c_void_p(buf.value + 4 * first), 4 * count)
+            got = L.download(buf, (n,))
+            expect = ones.copy()
+            expect[first:first + count] = 0.0
+            assert np.array_equal(got, expect), (first, count)
+        with pytest.raises(F.FastConvError):
+            L.fill_zero(ctypes.c_void_p(buf.value + 2), 8)          # not a 4-byte boundary
+    finally:
+        L.close()
