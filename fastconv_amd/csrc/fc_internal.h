@@ -73,8 +73,11 @@ int fc_igemm_ws_run(fc_context *ctx, const fc_igemm_plan *plan, int index, const
 // Called by the fc_wino_*onepass* entry points after they have checked plan and pointers.
 bool fc_wino_smallc_applies(const fc_conv_shape *s);
 int fc_wino_smallc_filter_transform(fc_context *ctx, const fc_wino_plan *plan, const float *w_dev, float *U_dev);
-int fc_wino_smallc_conv(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev, const float *U_dev,
+// w_dev == nullptr: U_dev holds the transformed filter; otherwise the kernel transforms w_dev itself and fills U_dev
+int fc_wino_smallc_conv(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev, float *U_dev, const float *w_dev,
                         const float *bias_dev, int relu, float *y_dev);
+// whether a forward call that has to transform the filter should leave that to the convolution kernel
+bool fc_wino_smallc_transforms_inside(const fc_context *ctx, const fc_wino_plan *plan);
 
 // Brackets one kernel launch with events when timing is on.
 struct fc_stage_scope {

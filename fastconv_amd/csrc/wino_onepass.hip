@@ -367,7 +367,8 @@ extern "C" int fc_wino_conv_onepass(fc_context *ctx, const fc_wino_plan *plan, c
     if (!y_dev) return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_conv_onepass: null output", hipSuccess);
     if (((uintptr_t)y_dev & 7) != 0 || ((uintptr_t)U_dev & 15) != 0 || ((uintptr_t)x_dev & 3) != 0)
         return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_conv_onepass: y must be 8-byte and U 16-byte aligned", hipSuccess);
-    if (fc_wino_smallc_applies(&plan->shape)) return fc_wino_smallc_conv(ctx, plan, x_dev, U_dev, bias_dev, relu, y_dev);
+    if (fc_wino_smallc_applies(&plan->shape))
+        return fc_wino_smallc_conv(ctx, plan, x_dev, const_cast<float *>(U_dev), nullptr, bias_dev, relu, y_dev);
     if (!ctx->onepass_lds_granted) {
         if (ctx->capturing)
             return fc_set_error(ctx, FC_ERR_STATE, "fc_wino_conv_onepass: run this kernel once before recording a graph with it", hipSuccess);
@@ -407,7 +408,18 @@ extern "C" int fc_wino_prefer_onepass(const fc_conv_shape *s) {
 extern "C" int fc_wino_forward_onepass(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev, const float *w_dev,
                                        const float *bias_dev, int relu, int filter_ready, float *U_dev, float *y_dev) {
     if (!filter_ready) {
-        const int rc = fc_wino_onepass_filter_transform(ctx, plan, w_dev, U_dev);
+        int rc = onepass_plan_check(ctx, plan, w_dev, U_dev);
+        if (rc) return rc;
+        if (fc_wino_smallc_applies(&plan->shape) && fc_wino_smallc_transforms_inside(ctx, plan)) {
+            // few tiles: one launch, the filter is transformed by the wavefronts that use it (and U filled all the same)
+            rc = onepass_plan_check(ctx, plan, x_dev, U_dev);
+            if (rc) return rc;
+            if (!y_dev) return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_forward_onepass: null output", hipSuccess);
+            if (((uintptr_t)y_dev & 7) != 0 || ((uintptr_t)U_dev & 15) != 0 || ((uintptr_t)x_dev & 3) != 0 || ((uintptr_t)w_dev & 3) != 0)
+                return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_forward_onepass: y must be 8-byte and U 16-byte aligned", hipSuccess);
+            return fc_wino_smallc_conv(ctx, plan, x_dev, U_dev, w_dev, bias_dev, relu, y_dev);
+        }
+        rc = fc_wino_onepass_filter_transform(ctx, plan, w_dev, U_dev);
         if (rc) return rc;
     }
     return fc_wino_conv_onepass(ctx, plan, x_dev, U_dev, bias_dev, relu, y_dev);

@@ -84,6 +84,53 @@ __device__ __forceinline__ UReg<C> load_ureg(const float *__restrict__ U, int k,
     return r;
 }
 
+// The same operand made from the 3x3 filter inside the convolution kernel (no filter-transform launch in front
+// of a layer with few tiles).  load_raw: lane e < 9*C fetches value e of the 9*C filter values of channel k
+// (zeros past the last channel).  make_ureg: lane f = 8 j + i turns them into U[k][i][j][c] = (G g G^T)[i][j];
+// row i of G applied as g8 applies it, ((a0*g0 + a2*g2) + a1*g1) * scale with coefficients 0, +-1, +-2, 4 whose
+// products are exact (what differs from wino_smallc_filter_kernel's values is where the compiler fuses a scale
+// into the addition that follows it: the last bit of some values).
+template <int C>
+__device__ __forceinline__ float load_raw(const float *__restrict__ w, int K, int k, int lane) {
+    const float *src = uniform_ptr(w + (size_t)min(k, K - 1) * (9 * C));
+    const float v = src[min(lane, 9 * C - 1)];
+    return (k < K && lane < 9 * C) ? v : 0.f;
+}
+
+struct GRow {
+    float a0, a2, a1, scale;
+};
+
+__device__ __forceinline__ GRow g_row(int i) {
+    const float c29 = (float)(-2.0 / 9), c90 = (float)(1.0 / 90), c180 = (float)(1.0 / 180);
+    GRow r;
+    r.a0 = i == 7 ? 0.f : (i == 5 || i == 6) ? 4.f : 1.f;
+    r.a2 = i == 0 ? 0.f : (i == 3 || i == 4) ? 4.f : 1.f;
+    r.a1 = (i == 0 || i == 7) ? 0.f : i == 1 ? 1.f : i == 2 ? -1.f : (i & 1) ? 2.f : -2.f;
+    r.scale = (i == 0 || i == 7) ? 1.f : i <= 2 ? c29 : i <= 4 ? c90 : c180;
+    return r;
+}
+
+__device__ __forceinline__ float g_apply(const GRow &r, float g0, float g1, float g2) {
+    return ((r.a0 * g0 + r.a2 * g2) + r.a1 * g1) * r.scale;
+}
+
+template <int C>
+__device__ __forceinline__ UReg<C> make_ureg(float raw, const GRow &gi, const GRow &gj) {
+    UReg<C> r;
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+        float g[9];
+#pragma unroll
+        for (int e = 0; e < 9; e++) g[e] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, raw), c * 9 + e));
+        float t[3];
+#pragma unroll
+        for (int b = 0; b < 3; b++) t[b] = g_apply(gi, g[b], g[3 + b], g[6 + b]);      // column b of the filter: rows 0, 1, 2
+        r.c[c] = g_apply(gj, t[0], t[1], t[2]);
+    }
+    return r;
+}
+
 // One tile column of one output channel: the eight products over the input channels and the
 // column half of the output transform.  The empty asm ties the results to this point of the
 // instruction stream (pure arithmetic is otherwise free to sink below the scheduling barrier
@@ -203,14 +250,18 @@ __device__ __forceinline__ void sc_step(const SmallCParams &p, const UReg<C> &u,
     }
 }
 
-template <int C, bool ROWST>
-__global__ __launch_bounds__(kScThreads) void wino_smallc_kernel(const float *__restrict__ x, const float *__restrict__ U,
-                                                                 const float *__restrict__ bias, float *__restrict__ y,
-                                                                 const SmallCParams p) {
+// RAWW: U_or_w is the untransformed filter [K][C][3][3]; every wavefront transforms the filters of its output
+// channels itself (a few dozen vector instructions per channel), and the workgroups of the first tile block
+// write them to Uout in the layout of wino_smallc_filter_kernel, so that U is filled as after that kernel.
+template <int C, bool ROWST, bool RAWW>
+__global__ __launch_bounds__(kScThreads) void wino_smallc_kernel(const float *__restrict__ x, const float *__restrict__ U_or_w,
+                                                                 float *__restrict__ Uout, const float *__restrict__ bias,
+                                                                 float *__restrict__ y, const SmallCParams p) {
     constexpr int TILES = sc_tiles(C);
     extern __shared__ float Vs[];   // [8 j][8 i][TILES][C], then one store buffer per wavefront
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const float *U = U_or_w;
     // workgroups are dealt to the eight XCDs in turn: give each XCD a contiguous range of tile
     // blocks, so that the cache lines two neighbouring blocks share meet in one L2
     const int tblk = (blockIdx.x & 7) * p.blocksPerXcd + (blockIdx.x >> 3);
@@ -223,6 +274,14 @@ __global__ __launch_bounds__(kScThreads) void wino_smallc_kernel(const float *__
     const uint32_t n = fc_div(band, p.divTH);
     const int th = (int)(band - n * (uint32_t)p.tH);
     const int vlane = min(lane, TILES - 1);
+    const int kpw = p.kPerBlock >> 2;
+    const int kFirst = blockIdx.y * p.kPerBlock + wave * kpw;
+    // RAWW: the filters of this wavefront's first two channels, asked for before anything else
+    float rawA = 0.f, rawB = 0.f;
+    if (RAWW) {
+        rawA = load_raw<C>(U_or_w, p.K, kFirst, lane);
+        rawB = load_raw<C>(U_or_w, p.K, kFirst + 1, lane);
+    }
 
     // ---- input transform of channel `wave` of this lane's tile.  The patch is read through a
     // buffer resource: an element outside the image gets an offset past the end of x and the
@@ -268,9 +327,23 @@ __global__ __launch_bounds__(kScThreads) void wino_smallc_kernel(const float *__
     // outputs of a channel are finished and stored during the step of the next one.  (p.zero is
     // 0: it ties the LDS addresses to the loop counter, or all 64 x C values of the transformed
     // patch would be kept in registers across the loop.)
-    const int kpw = p.kPerBlock >> 2;
-    const int kFirst = blockIdx.y * p.kPerBlock + wave * kpw;
     const int kCount = min(kpw, p.K - kFirst);
+    const GRow gi = g_row(lane & 7), gj = g_row(lane >> 3);
+    // RAWW, first tile block: row k of U as wino_smallc_filter_kernel lays it out, [8 j][8 i][4 c]; channels C..3 and
+    // the rows of the padding K..K_pad-1 are zeros
+    auto keep = [&](int k, const UReg<C> &u) {
+        if (RAWW && tblk == 0 && k < kFirst + kpw) {
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            v.x = u.c[0];
+            if (C > 1) v.y = u.c[C > 1 ? 1 : 0];
+            if (C > 2) v.z = u.c[C > 2 ? 2 : 0];
+            if (C > 3) v.w = u.c[C > 3 ? 3 : 0];
+            *reinterpret_cast<float4 *>(Uout + (size_t)k * 256 + lane * 4) = v;
+        }
+    };
+    if (RAWW && tblk == 0)
+        for (int k = kFirst + max(kCount, 0); k < kFirst + kpw; k++)
+            *reinterpret_cast<float4 *>(Uout + (size_t)k * 256 + lane * 4) = make_float4(0.f, 0.f, 0.f, 0.f);
     if (kCount <= 0) return;
     // ReLU as a maximum with 0, no ReLU as a maximum with -inf: one v_maximum3_f32 either way, which keeps a NaN
     const float floorv = p.relu ? 0.f : -__builtin_inff();
@@ -297,15 +370,26 @@ __global__ __launch_bounds__(kScThreads) void wino_smallc_kernel(const float *__
     const float *vlanep = Vs + vlane * C;
     const int kMax = p.K_pad - 1;   // the filter of a channel is fetched one step ahead; never past the padded end
     float ra[6][8], rb[6][8];
-    UReg<C> ua = load_ureg<C>(U, kFirst, lane), ub = load_ureg<C>(U, min(kFirst + 1, kMax), lane);
+    // the operand of channel k: from U, or (RAWW) from the filter values fetched two channels ahead, whose register
+    // then takes the values of the channel two further on
+    auto operand = [&](int k, float &raw) {
+        if (RAWW) {
+            const UReg<C> u = make_ureg<C>(raw, gi, gj);
+            raw = load_raw<C>(U_or_w, p.K, k + 2, lane);
+            if (k < p.K) keep(k, u);
+            return u;
+        }
+        return load_ureg<C>(U, min(k, kMax), lane);
+    };
+    UReg<C> ua = operand(kFirst, rawA), ub = operand(kFirst + 1, rawB);
     sc_step<C, ROWST, true, false>(p, ua, bias, y, vlanep, st, lane, 0, 0, floorv, ra, rb);
     int kk = 1;
     for (; kk + 1 < kCount; kk += 2) {
         const int tie = kk * p.zero, tie2 = (kk + 1) * p.zero;   // one per step: equal addresses would be read once
         const int k = __builtin_amdgcn_readfirstlane(kFirst + kk);
-        ua = load_ureg<C>(U, k + 1, lane);
+        ua = operand(k + 1, rawA);
         sc_step<C, ROWST, true, true>(p, ub, bias, y, vlanep + tie, st, lane, k - 1, tie, floorv, rb, ra);
-        ub = load_ureg<C>(U, min(k + 2, kMax), lane);
+        ub = operand(k + 2, rawB);
         sc_step<C, ROWST, true, true>(p, ua, bias, y, vlanep + tie2, st, lane, k, tie2, floorv, ra, rb);
     }
     const int kLast = __builtin_amdgcn_readfirstlane(kFirst + kCount - 1);
@@ -333,7 +417,23 @@ int fc_wino_smallc_filter_transform(fc_context *ctx, const fc_wino_plan *plan, c
     return FC_OK;
 }
 
-int fc_wino_smallc_conv(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev, const float *U_dev,
+// Output channels per workgroup: 64 when that still gives every CU a few workgroups, else 16, or 8 when even
+// that leaves CUs without one (batch 1)
+static int sc_k_per_block(const fc_context *ctx, const fc_wino_plan *plan) {
+    const int tiles = sc_tiles(plan->shape.C);
+    const long tileBlocks = (plan->T + tiles - 1) / tiles;
+    const long cus = ctx->props.multiProcessorCount;
+    return tileBlocks * (plan->K_pad / 64) >= 2 * cus ? 64 : tileBlocks * (plan->K_pad / 16) >= cus ? 16 : 8;
+}
+
+// Where a wavefront has only a few output channels the filter transform is cheaper inside the convolution kernel
+// than as a launch in front of it (4.5 us plus the gap between two launches; the whole layer takes 13 us at batch 1).
+bool fc_wino_smallc_transforms_inside(const fc_context *ctx, const fc_wino_plan *plan) {
+    return sc_k_per_block(ctx, plan) < 64 && ((size_t)plan->shape.K * plan->shape.C * 9) < ((size_t)1 << 29);
+}
+
+// w_dev == nullptr: U_dev holds the transformed filter.  Otherwise the kernel transforms w_dev itself and fills U_dev.
+int fc_wino_smallc_conv(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev, float *U_dev, const float *w_dev,
                         const float *bias_dev, int relu, float *y_dev) {
     const fc_conv_shape &s = plan->shape;
     SmallCParams p;
@@ -347,10 +447,7 @@ int fc_wino_smallc_conv(fc_context *ctx, const fc_wino_plan *plan, const float *
     p.divTH = fc_make_fastdiv(p.tH);
     const int tiles = sc_tiles(s.C);
     const long tileBlocks = (plan->T + tiles - 1) / tiles;
-    // 64 output channels per workgroup when that still gives every CU a few workgroups, else 16, or 8 when even
-    // that leaves CUs without one (batch 1)
-    const long cus = ctx->props.multiProcessorCount;
-    p.kPerBlock = tileBlocks * (plan->K_pad / 64) >= 2 * cus ? 64 : tileBlocks * (plan->K_pad / 16) >= cus ? 16 : 8;
+    p.kPerBlock = sc_k_per_block(ctx, plan);
     const long gy = plan->K_pad / p.kPerBlock;
     if (tileBlocks >= (1l << 31) - 8 || gy > 65535)
         return fc_set_error(ctx, FC_ERR_UNSUPPORTED, "fc_wino_conv_onepass: grid too large", hipSuccess);
@@ -364,17 +461,24 @@ int fc_wino_smallc_conv(fc_context *ctx, const fc_wino_plan *plan, const float *
     if (lds > 64 * 1024 && !ctx->smallc_lds_granted) {   // four channels: 70 KiB
         if (ctx->capturing)
             return fc_set_error(ctx, FC_ERR_STATE, "fc_wino_conv_onepass: run this kernel once before recording a graph with it", hipSuccess);
-        FC_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)wino_smallc_kernel<4, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        FC_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)wino_smallc_kernel<4, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        FC_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)wino_smallc_kernel<4, true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        FC_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)wino_smallc_kernel<4, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        FC_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)wino_smallc_kernel<4, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        FC_HIP_CHECK(ctx, hipFuncSetAttribute((const void *)wino_smallc_kernel<4, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         ctx->smallc_lds_granted = true;
     }
     fc_stage_scope scope(ctx, FC_STAGE_ONEPASS);
+#define FC_SC_LAUNCH2(C_, ROWST_)                                                                                \
+    do {                                                                                                         \
+        if (w_dev)                                                                                               \
+            wino_smallc_kernel<C_, ROWST_, true><<<grid, dim3(kScThreads), lds, ctx->stream>>>(x_dev, w_dev, U_dev, bias_dev, y_dev, p);   \
+        else                                                                                                     \
+            wino_smallc_kernel<C_, ROWST_, false><<<grid, dim3(kScThreads), lds, ctx->stream>>>(x_dev, U_dev, nullptr, bias_dev, y_dev, p); \
+    } while (0)
 #define FC_SC_LAUNCH(C_)                                                                                         \
     do {                                                                                                         \
-        if (rowStores)                                                                                           \
-            wino_smallc_kernel<C_, true><<<grid, dim3(kScThreads), lds, ctx->stream>>>(x_dev, U_dev, bias_dev, y_dev, p);  \
-        else                                                                                                     \
-            wino_smallc_kernel<C_, false><<<grid, dim3(kScThreads), lds, ctx->stream>>>(x_dev, U_dev, bias_dev, y_dev, p); \
+        if (rowStores) FC_SC_LAUNCH2(C_, true);                                                                  \
+        else FC_SC_LAUNCH2(C_, false);                                                                           \
     } while (0)
     switch (s.C) {
     case 1: FC_SC_LAUNCH(1); break;
@@ -384,6 +488,7 @@ int fc_wino_smallc_conv(fc_context *ctx, const fc_wino_plan *plan, const float *
     default: return fc_set_error(ctx, FC_ERR_INVALID, "fc_wino_conv_onepass: more than four input channels", hipSuccess);
     }
 #undef FC_SC_LAUNCH
+#undef FC_SC_LAUNCH2
     FC_LAUNCH_CHECK(ctx, "wino_smallc_kernel");
     return FC_OK;
 }

@@ -352,6 +352,45 @@ def test_winograd_small_channel_kernel(lib, shp, pads):
     assert O.max_rel_err(y2, O.naive_conv_f64(s, x, w)) <= TOL_WINO
 
 
+@pytest.mark.parametrize("shp", [(1, 3, 224, 224, 64), (1, 1, 20, 20, 1), (2, 2, 31, 40, 17), (1, 4, 64, 64, 130),
+                                 (2, 3, 44, 46, 70), (1, 3, 30, 30, 9), (32, 3, 64, 64, 64)])
+def test_winograd_small_channel_kernel_transforms_the_filter_itself(lib, shp):
+    """With few tiles fc_wino_forward_onepass leaves the filter transform to the convolution kernel (one
+    launch): the output and the U it leaves behind are those of fc_wino_onepass_filter_transform followed by
+    fc_wino_conv_onepass (to rounding), rows and channels of the padding included; a second call with
+    filter_ready reads that U and gives the same bits.  (The last shape has enough tiles for the two-launch path.)"""
+    s = O.shape(*shp)
+    cs = cshape(s)
+    x, w = O.make_inputs(s, seed=shp[4] + 5)
+    bias = O.rng_uniform(4, (s.K,))
+    announce("small-channel winograd, filter transformed in the kernel", shp)
+    plan = lib.wino_onepass_plan(cs)
+    nU = plan.U_bytes // 4
+    mark = lib.mark()
+    try:
+        dx, dw, db = lib.upload(x), lib.upload(w), lib.upload(bias)
+        poison = np.full(nU, 7.0, np.float32)
+        U1, U2 = lib.upload(poison), lib.upload(poison)
+        y = lib.alloc(4 * s.N * s.K * plan.OH * plan.OW)
+        lib.wino_onepass_filter_transform(plan, dw, U1)
+        lib.wino_conv_onepass(plan, dx, U1, y, db, True)
+        y1 = lib.download(y, (s.N, s.K, plan.OH, plan.OW))
+        lib.fill_zero(y, 4 * s.N * s.K * plan.OH * plan.OW)
+        lib.wino_forward_onepass(plan, dx, dw, U2, y, db, True)
+        y2 = lib.download(y, (s.N, s.K, plan.OH, plan.OW))
+        # the same formulas, but the compiler fuses multiplications and additions differently in the two kernels
+        assert O.max_rel_err(y2, y1) <= 2e-6
+        Ua, Ub = lib.download(U1, (nU,)), lib.download(U2, (nU,))
+        assert np.abs(Ua - Ub).max() <= 1e-6 * np.abs(Ua).max()
+        assert np.array_equal(Ua == 0.0, Ub == 0.0)          # the zeros of the padding, and nothing left of the 7s
+        lib.fill_zero(y, 4 * s.N * s.K * plan.OH * plan.OW)
+        lib.wino_forward_onepass(plan, dx, dw, U2, y, db, True, filter_ready=True)
+        assert np.array_equal(lib.download(y, (s.N, s.K, plan.OH, plan.OW)), y2)
+    finally:
+        lib.release(mark)
+    assert O.max_rel_err(y1, np.maximum(O.naive_conv_f64(s, x, w, bias), 0.0)) <= TOL_WINO
+
+
 def test_winograd_single_kernel_full_size_layers(lib):
     for (N, C, H, K) in [(32, 3, 224, 64), (32, 64, 112, 128), (8, 64, 224, 64), (32, 64, 224, 64)]:
         s = O.shape(N, C, H, H, K)
