@@ -300,7 +300,10 @@ int fc_wino_onepass_filter_transform(fc_context *ctx, const fc_wino_plan *plan,
 int fc_wino_conv_onepass(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev,
                          const float *U_dev, const float *bias_dev, int relu, float *y_dev);
 
-/* Filter transform (unless filter_ready) + fc_wino_conv_onepass. */
+/* Filter transform (unless filter_ready) + fc_wino_conv_onepass.  U_dev holds the transformed filter
+ * afterwards either way; for a layer with at most four input channels and few tiles the two run as one
+ * launch (the convolution kernel transforms the filter itself and writes U_dev as a by-product, equal to
+ * fc_wino_onepass_filter_transform's to the last bit or two). */
 int fc_wino_forward_onepass(fc_context *ctx, const fc_wino_plan *plan, const float *x_dev,
                             const float *w_dev, const float *bias_dev, int relu, int filter_ready,
                             float *U_dev, float *y_dev);
