@@ -161,3 +161,13 @@ def test_bench_reads_measured_traffic_from_the_committed_profile():
         assert 0.95 <= table[key] / algorithmic <= 1.25, (key, table[key] / algorithmic)
         seen += 1
     assert seen >= 5
+
+
+def test_bench_refuses_more_than_one_gpu_with_a_message():
+    """bench.py --gpus N with N above 1 exits before touching the GPU and says why."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in r.stderr and r.stdout.strip() == ""
