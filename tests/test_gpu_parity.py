@@ -379,7 +379,7 @@ def test_winograd_small_channel_kernel_transforms_the_filter_itself(lib, shp):
         lib.wino_forward_onepass(plan, dx, dw, U2, y, db, True)
         y2 = lib.download(y, (s.N, s.K, plan.OH, plan.OW))
         # the same formulas, but the compiler fuses multiplications and additions differently in the two kernels
-        assert O.max_rel_err(y2, y1) <= 2e-6
+        assert O.max_rel_err(y2, y1) <= 1e-5
         Ua, Ub = lib.download(U1, (nU,)), lib.download(U2, (nU,))
         assert np.abs(Ua - Ub).max() <= 1e-6 * np.abs(Ua).max()
         assert np.array_equal(Ua == 0.0, Ub == 0.0)          # the zeros of the padding, and nothing left of the 7s
